@@ -1,0 +1,217 @@
+"""Pins for the CPU oracle: each check is independent of the oracle's own formulae
+(a third-party implementation, a brute-force loop, or a closed form / invariant)."""
+import math
+
+import pytest
+import torch
+
+from oracle import neox_oracle as O
+from oracle.neox_oracle import NeoxDims
+
+TINY = NeoxDims(hidden=64, heads=4, head_dim=16, rotary_dim=4, ffn=256)
+SMALL = NeoxDims(hidden=256, heads=8, head_dim=32, rotary_dim=8, ffn=1024)
+
+
+def _mk(dims, S, seed=0, w_std=0.05):
+    w = O.make_layer_weights(dims, layer=seed, w_std=w_std, b_std=0.05)
+    x, k, v, cos, sin = O.make_layer_inputs(dims, S, capacity=S + 2, seed=seed)
+    return w, x, k, v, cos, sin
+
+
+# ---------------------------------------------------------------- HF GPTNeoXLayer (third party)
+@pytest.mark.parametrize("dims,S", [(TINY, 5), (SMALL, 33), (SMALL, 0),
+                                    (NeoxDims(320, 4, 80, 20, 1280), 17)])
+def test_layer_matches_hf_gptneox_layer(dims, S):
+    from oracle import hf_neox
+    w, x, k, v, cos, sin = _mk(dims, S)
+    r = O.neox_layer_decode(x, w, k, v, cos, sin, S, dims, dtype=torch.float64, round_io=False)
+    layer = hf_neox.build_hf_layer(dims, w, dtype=torch.float64)
+    out, k_new, v_new = hf_neox.hf_layer_decode(layer, x, k, v, cos, sin, S, dims, dtype=torch.float64)
+    # HF's eager attention runs its softmax in float32 even for a float64 module: ~1e-8 noise
+    assert torch.allclose(r["output"], out, atol=1e-6, rtol=0)
+    assert torch.allclose(r["k_new"], k_new, atol=1e-12, rtol=0)
+    assert torch.allclose(r["v_new"], v_new, atol=1e-12, rtol=0)
+
+
+def test_rope_table_matches_hf_rotary_embedding():
+    from oracle import hf_neox
+    from transformers.models.gpt_neox.modeling_gpt_neox import GPTNeoXRotaryEmbedding
+    dims = NeoxDims(320, 4, 80, 20, 1280)
+    rot = GPTNeoXRotaryEmbedding(hf_neox._config(dims))
+    pos = torch.tensor([[0, 1, 7, 513, 4095]])
+    c, s = rot(torch.zeros(1, 5, dims.hidden), pos)
+    c2, s2 = O.rope_table(pos[0], dims.rotary_dim)
+    assert c.shape[-1] == dims.rotary_dim
+    # HF forms position*inv_freq in float32 (angle error ~ pos * 6e-8); the oracle uses float64 angles
+    assert torch.allclose(c[0, :3], c2[:3], atol=2e-6) and torch.allclose(s[0, :3], s2[:3], atol=2e-6)
+    assert torch.allclose(c[0], c2, atol=1e-3) and torch.allclose(s[0], s2, atol=1e-3)
+
+
+def test_stack_matches_hf_causal_lm():
+    from oracle import hf_neox
+    from transformers import DynamicCache
+    dims, L, V, S = TINY, 3, 97, 6
+    layers = [O.make_layer_weights(dims, layer=i, w_std=0.08, b_std=0.05) for i in range(L)]
+    g = torch.Generator().manual_seed(7)
+    embed = torch.randn((V, dims.hidden), generator=g).half()
+    lm = (torch.randn((V, dims.hidden), generator=g) * 0.1).half()
+    fw = (1 + 0.02 * torch.randn(dims.hidden, generator=g)).half()
+    fb = (0.01 * torch.randn(dims.hidden, generator=g)).half()
+    kcs = [torch.randn((S + 2, dims.hidden), generator=g).half() for _ in range(L)]
+    vcs = [torch.randn((S + 2, dims.hidden), generator=g).half() for _ in range(L)]
+    model = hf_neox.build_hf_model(dims, layers, embed, fw, fb, lm, dtype=torch.float64)
+    nh, D = dims.heads, dims.head_dim
+    past = DynamicCache(ddp_cache_data=[
+        (kc[:S].double().reshape(S, nh, D).permute(1, 0, 2)[None].contiguous(),
+         vc[:S].double().reshape(S, nh, D).permute(1, 0, 2)[None].contiguous()) for kc, vc in zip(kcs, vcs)])
+    tok = 11
+    with torch.no_grad():
+        hf = model(input_ids=torch.tensor([[tok]]), past_key_values=past,
+                   position_ids=torch.tensor([[S]]), use_cache=True).logits[0, -1]
+    r = O.neox_stack_decode(tok, embed, layers, fw, fb, lm, [k.clone() for k in kcs], [v.clone() for v in vcs],
+                            S, dims, dtype=torch.float64)
+    # the oracle rounds the hidden state to fp16 between layers (that is what the op API carries)
+    assert torch.allclose(r["logits"], hf, atol=5e-3)
+    assert r["next_token"] == int(hf.argmax())
+
+
+# ---------------------------------------------------------------- brute force, pure Python float64
+def _brute_force_layer(x, w, kc, vc, cos, sin, S, d):
+    H, nh, D, rot, F = d.hidden, d.heads, d.head_dim, d.rotary_dim, d.ffn
+    xs = [float(t) for t in x.reshape(-1)]
+    mean = sum(xs) / H
+    var = sum((t - mean) ** 2 for t in xs) / H
+    rstd = 1.0 / math.sqrt(var + d.eps)
+    L = lambda name: w[name].double().reshape(-1).tolist()
+    M = lambda name: w[name].double().tolist()
+    ln1 = [(xs[i] - mean) * rstd * L("ln_w")[i] + L("ln_b")[i] for i in range(H)]
+    ln2 = [(xs[i] - mean) * rstd * L("post_ln_w")[i] + L("post_ln_b")[i] for i in range(H)]
+    Wq, bq = M("w_qkv"), L("b_qkv")
+    qkv = [sum(Wq[r][c] * ln1[c] for c in range(H)) + bq[r] for r in range(3 * H)]
+    cs, sn = cos.double().reshape(-1).tolist(), sin.double().reshape(-1).tolist()
+
+    def rope(vec):
+        o = list(vec)
+        for i in range(rot // 2):
+            a, b = vec[i], vec[i + rot // 2]
+            o[i] = a * cs[i] - b * sn[i]
+            o[i + rot // 2] = b * cs[i + rot // 2] + a * sn[i + rot // 2]
+        return o
+
+    attn_in = []
+    k_new, v_new = [], []
+    for h in range(nh):
+        base = h * 3 * D
+        q = rope(qkv[base:base + D])
+        k = rope(qkv[base + D:base + 2 * D])
+        v = qkv[base + 2 * D:base + 3 * D]
+        k_new.append(k)
+        v_new.append(v)
+        keys = [kc[s, h * D:(h + 1) * D].double().tolist() for s in range(S)] + [k]
+        vals = [vc[s, h * D:(h + 1) * D].double().tolist() for s in range(S)] + [v]
+        sc = [sum(q[i] * kk[i] for i in range(D)) / math.sqrt(D) for kk in keys]
+        m = max(sc)
+        e = [math.exp(t - m) for t in sc]
+        z = sum(e)
+        attn_in += [sum(e[s] * vals[s][i] for s in range(S + 1)) / z for i in range(D)]
+    Wo, bo = M("w_o"), L("b_o")
+    attn = [sum(Wo[r][c] * attn_in[c] for c in range(H)) + bo[r] for r in range(H)]
+    Wu, bu = M("w_up"), L("b_up")
+    up = [sum(Wu[r][c] * ln2[c] for c in range(H)) + bu[r] for r in range(F)]
+    g = [0.5 * t * (1 + math.tanh(math.sqrt(2 / math.pi) * (t + 0.044715 * t ** 3))) for t in up]
+    Wd, bd = M("w_down"), L("b_down")
+    out = [xs[r] + attn[r] + sum(Wd[r][c] * g[c] for c in range(F)) + bd[r] for r in range(H)]
+    return out, k_new, v_new
+
+
+def test_layer_matches_pure_python_brute_force():
+    d, S = TINY, 5
+    w, x, k, v, cos, sin = _mk(d, S, seed=3, w_std=0.1)
+    out, k_new, v_new = _brute_force_layer(x, w, k, v, cos, sin, S, d)
+    r = O.neox_layer_decode(x, w, k, v, cos, sin, S, d, dtype=torch.float64, round_io=False)
+    assert torch.allclose(r["output"].reshape(-1), torch.tensor(out, dtype=torch.float64), atol=1e-10)
+    assert torch.allclose(r["k_new"].reshape(-1), torch.tensor(k_new, dtype=torch.float64).reshape(-1), atol=1e-12)
+    assert torch.allclose(r["v_new"].reshape(-1), torch.tensor(v_new, dtype=torch.float64).reshape(-1), atol=1e-12)
+
+
+# ---------------------------------------------------------------- closed forms and invariants
+def test_layer_norm_against_torch_and_constant_vector():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(3, 96, generator=g, dtype=torch.float64)
+    w, b = torch.randn(96, generator=g, dtype=torch.float64), torch.randn(96, generator=g, dtype=torch.float64)
+    assert torch.allclose(O.layer_norm(x, w, b, 1e-5), torch.nn.functional.layer_norm(x, (96,), w, b, 1e-5), atol=1e-12)
+    assert torch.allclose(O.layer_norm(torch.full((1, 96), 3.25, dtype=torch.float64), w, b, 1e-5), b[None], atol=1e-12)
+
+
+def test_gelu_against_torch():
+    x = torch.linspace(-12, 12, 4001, dtype=torch.float64)
+    assert torch.allclose(O.gelu_tanh(x), torch.nn.functional.gelu(x, approximate="tanh"), atol=1e-12)
+
+
+def test_rope_identity_norm_and_passthrough():
+    g = torch.Generator().manual_seed(2)
+    t = torch.randn(4, 16, generator=g, dtype=torch.float64)
+    one, zero = torch.ones(8), torch.zeros(8)
+    assert torch.equal(O.rope_partial_neox(t, one, zero, 8), t)
+    c0, s0 = O.rope_table(torch.tensor([0]), 8)
+    assert torch.allclose(O.rope_partial_neox(t, c0, s0, 8), t, atol=1e-12)
+    c, s = O.rope_table(torch.tensor([37]), 8, dtype=torch.float64)
+    r = O.rope_partial_neox(t, c, s, 8)
+    assert torch.equal(r[:, 8:], t[:, 8:])
+    for i in range(4):   # pairs (i, i+4) are rotated: norm preserved
+        assert torch.allclose(r[:, i] ** 2 + r[:, i + 4] ** 2, t[:, i] ** 2 + t[:, i + 4] ** 2, atol=1e-12)
+    # sign convention: rotating e_0 by angle theta gives (cos, sin) on dims (0, rot/2)
+    e = torch.zeros(1, 16, dtype=torch.float64); e[0, 0] = 1
+    r = O.rope_partial_neox(e, c, s, 8)
+    assert math.isclose(r[0, 0], math.cos(37.0)) and math.isclose(r[0, 4], math.sin(37.0))
+
+
+def test_zero_weights_give_identity_and_bias_only():
+    d, S = SMALL, 9
+    w, x, k, v, cos, sin = _mk(d, S)
+    z = {n: torch.zeros_like(t) for n, t in w.items()}
+    z["ln_w"], z["post_ln_w"] = w["ln_w"], w["post_ln_w"]
+    r = O.neox_layer_decode(x, z, k, v, cos, sin, S, d)
+    assert torch.equal(r["output"].half(), x)
+    z["b_o"], z["b_down"] = w["b_o"], w["b_down"]
+    r = O.neox_layer_decode(x, z, k, v, cos, sin, S, d, dtype=torch.float64, round_io=False)
+    assert torch.allclose(r["output"], x.double() + w["b_o"].double() + w["b_down"].double(), atol=1e-12)
+
+
+def test_attention_special_cases():
+    d = SMALL
+    w, x, k, v, cos, sin = _mk(d, 0)
+    r = O.neox_layer_decode(x, w, k, v, cos, sin, 0, d, dtype=torch.float64, round_io=False)
+    assert torch.allclose(r["attn_heads"], r["v_new"][0], atol=1e-12)          # S=0: only the new token
+    S = 12
+    w, x, k, v, cos, sin = _mk(d, S)
+    r0 = O.neox_layer_decode(x, w, k, v, cos, sin, S, d, dtype=torch.float64, round_io=False)
+    k[:S] = r0["k_new"].reshape(1, -1).half()                                  # all keys identical -> mean of V
+    r = O.neox_layer_decode(x, w, k, v, cos, sin, S, d, dtype=torch.float64, round_io=True)
+    mean_v = (v[:S].double().sum(0) + r["v_new"].reshape(-1)) / (S + 1)
+    assert torch.allclose(r["attn_heads"].reshape(-1), mean_v, atol=1e-9)
+    # permutation invariance over cache rows and independence from rows >= S
+    w, x, k, v, cos, sin = _mk(d, S)
+    perm = torch.randperm(S, generator=torch.Generator().manual_seed(0))
+    k2, v2 = k.clone(), v.clone()
+    k2[:S], v2[:S] = k[perm], v[perm]
+    k2[S:], v2[S:] = -7.0, 123.0
+    a = O.neox_layer_decode(x, w, k, v, cos, sin, S, d, dtype=torch.float64)["output"]
+    b = O.neox_layer_decode(x, w, k2, v2, cos, sin, S, d, dtype=torch.float64)["output"]
+    assert torch.allclose(a, b, atol=1e-12)
+    # a dominant key selects its V row
+    k3 = k.clone()
+    q = r0["q"]
+    k3[3] = (q.reshape(-1) * 50).half()
+    r = O.neox_layer_decode(x, w, k3, v, cos, sin, S, d, dtype=torch.float64, round_io=False)
+    assert torch.allclose(r["attn_heads"].reshape(-1), v[3].double(), atol=1e-6)
+
+
+def test_cache_side_effect():
+    d, S = SMALL, 7
+    w, x, k, v, cos, sin = _mk(d, S)
+    k0, v0 = k.clone(), v.clone()
+    r = O.neox_layer_decode(x, w, k, v, cos, sin, S, d, write_cache=True)
+    assert torch.equal(k[S], r["k_new"].reshape(-1).half()) and torch.equal(v[S], r["v_new"].reshape(-1).half())
+    keep = [i for i in range(k.shape[0]) if i != S]
+    assert torch.equal(k[keep], k0[keep]) and torch.equal(v[keep], v0[keep])
