@@ -1,0 +1,73 @@
+"""In-tree build of the two native libraries (no JIT cache, no install step):
+
+  libcfpp.so          HIP kernels + the C ABI of include/cfpp.h, compiled by hipcc for gfx950
+  _clusterfusion.so   the PyTorch binding (host C++ only), compiled by g++ against libtorch
+
+Both land next to this file so that they travel with the source tree.
+`python -m clusterfusionplus_amd.build` rebuilds both.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+import sysconfig
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+INCLUDE = os.path.join(ROOT, "include")
+LIB = os.path.join(PKG, "libcfpp.so")
+EXT = os.path.join(PKG, "_clusterfusion.so")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # packed-fp32 arithmetic stays off in device code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd):
+    print("+ " + " ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if out.strip():
+        print(out, flush=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"build command failed ({res.returncode}): {' '.join(cmd)}")
+
+
+def build_lib():
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    _run([hipcc, *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", os.path.join(CSRC, "cfpp_kernels.hip"), "-o", LIB])
+    return LIB
+
+
+def build_ext():
+    import torch
+    from torch.utils import cpp_extension as ce
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    incs = [f"-I{p}" for p in ce.include_paths("cuda")] + [f"-I{sysconfig.get_paths()['include']}", f"-I{INCLUDE}"]
+    abi = int(torch.compiled_with_cxx11_abi())
+    cmd = [
+        "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wno-attributes",
+        "-DUSE_ROCM", "-D__HIP_PLATFORM_AMD__=1", "-DTORCH_EXTENSION_NAME=_clusterfusion",
+        "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
+        *incs, os.path.join(CSRC, "cfpp_torch.cpp"), "-o", EXT,
+        f"-L{PKG}", "-lcfpp", f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+        "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}",
+    ]
+    _run(cmd)
+    return EXT
+
+
+def build_all():
+    build_lib()
+    build_ext()
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

@@ -1,0 +1,790 @@
+// Kernels and C-ABI entry points of the GPT-NeoX decode step for MI355X (gfx950).
+// The device building blocks and the design overview live in cfpp_device.hpp.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <utility>
+#include <vector>
+
+#include "cfpp.h"
+#include "cfpp_device.hpp"
+
+using namespace cfpp;
+
+// =================================================================================================
+// kernels
+// =================================================================================================
+namespace {
+
+// ---- split mode: one launch per stage ----------------------------------------------------------
+template <int NCH, int NWV>
+__global__ __launch_bounds__(NWV * 64) void k_stage_a(LayerParams p, int do_qkv, int do_up) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int gw = blockIdx.x * NWV + wave, nw = gridDim.x * NWV;
+    half2_t x1[NCH][4], x2[NCH][4];
+    load_ln_pair<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, lane, x1, x2);
+    if (do_qkv) stage_a_qkv<NCH>(p, x1, gw, nw, lane);
+    if (do_up) stage_a_up<NCH>(p, x2, gw, nw, lane);
+}
+
+__global__ __launch_bounds__(256) void k_stage_b(LayerParams p) {
+    __shared__ AttnShared sh;
+    const int S = load_seq_len(p);
+    const int nitems = p.heads * p.nsplit;
+    for (int item = blockIdx.x; item < nitems; item += gridDim.x)
+        attention_item(p, item / p.nsplit, item % p.nsplit, S, sh);
+}
+
+template <int CPW, int NWV>
+__global__ __launch_bounds__(NWV * 64) void k_stage_c(LayerParams p, int KS, int RG) {
+    __shared__ StageCShared sh;
+    const StageC c = make_stage_c(p);
+    stage_c_rows<CPW>(c, blockIdx.x, gridDim.x, KS, RG, sh);
+}
+
+// ---- fused mode: one persistent launch ---------------------------------------------------------
+// Timeline of every workgroup (NW = total waves in the grid):
+//   LN -> QKV rows -> [arrive, per wave] -> MLP-up rows -> wait(epoch 1: all QKV rows written;
+//   the wait is hidden behind the MLP-up rows) -> attention items -> [arrive] -> wait(epoch 2)
+//   -> stage C rows -> exit counter (the last workgroup resets the counters for the next launch).
+// All workgroups must be co-resident: the host launches at most one per compute unit.
+template <int NCH, int CPW, int NWV>
+__global__ __launch_bounds__(NWV * 64) void k_fused(LayerParams p, int KS, int RG) {
+    __shared__ AttnShared sha;
+    __shared__ StageCShared shc;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int G = gridDim.x, gw = blockIdx.x * NWV + wave, nw = G * NWV;
+    int* epoch = p.bar;
+    int* exitc = p.bar + 1;
+    int* status = p.bar + 2;
+    const int S = load_seq_len(p);
+    {
+        half2_t x1[NCH][4], x2[NCH][4];
+        load_ln_pair<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, lane, x1, x2);
+        stage_a_qkv<NCH>(p, x1, gw, nw, lane);
+        if (lane == 0) counter_add_release(epoch, 1);
+        stage_a_up<NCH>(p, x2, gw, nw, lane);
+    }
+    grid_wait(epoch, nw, status);
+    const int nitems = p.heads * p.nsplit;
+    for (int item = blockIdx.x; item < nitems; item += G)
+        attention_item(p, item / p.nsplit, item % p.nsplit, S, sha);
+    __syncthreads();
+    if (threadIdx.x == 0) counter_add_release(epoch, NWV);
+    grid_wait(epoch, 2 * nw, status);
+    {
+        const StageC c = make_stage_c(p);
+        stage_c_rows<CPW>(c, blockIdx.x, G, KS, RG, shc);
+    }
+    if (threadIdx.x == 0) {
+        const int old = __hip_atomic_fetch_add(exitc, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if (old == G - 1) {
+            __hip_atomic_store(epoch, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(exitc, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+// ---- whole-model helpers -----------------------------------------------------------------------
+// hidden <- embed[token]
+__global__ void k_embed(const half_t* __restrict__ embed, const int* __restrict__ state, int H, int vocab,
+                        half_t* __restrict__ hidden) {
+    int tok = state[0];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (i < H) *reinterpret_cast<u32x4*>(hidden + i) = ld16(embed + (size_t)tok * H + i);
+}
+
+// logits = W LN(x); every workgroup also records its best (value, index) for the greedy pick
+template <int NCH, int NWV>
+__global__ __launch_bounds__(NWV * 64) void k_lm_head(const half_t* __restrict__ x, int H, float eps,
+                                                      const half_t* __restrict__ ln_w, const half_t* __restrict__ ln_b,
+                                                      const half_t* __restrict__ W, int vocab, float* __restrict__ logits,
+                                                      float* __restrict__ best_val, int* __restrict__ best_idx) {
+    __shared__ float sv[NWV];
+    __shared__ int si[NWV];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int gw = blockIdx.x * NWV + wave, nw = gridDim.x * NWV;
+    half2_t x1[NCH][4], x2[NCH][4];
+    load_ln_pair<NCH>(x, H, eps, ln_w, ln_b, nullptr, nullptr, lane, x1, x2);
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    gemv_rows_auto<NCH>(W, H, gw, nw, vocab, x1, lane, [&](int) { return 0.f; },
+                        [&](int r, float v, float) {
+                            if (lane == 0) logits[r] = v;
+                            if (v > bv || (v == bv && r < bi)) { bv = v; bi = r; }
+                        });
+    if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < NWV; ++w)
+            if (sv[w] > bv || (sv[w] == bv && si[w] < bi)) { bv = sv[w]; bi = si[w]; }
+        if (best_val) { best_val[blockIdx.x] = bv; best_idx[blockIdx.x] = bi; }
+    }
+}
+
+// token <- argmax, seq_len <- seq_len + 1, history[step] <- token
+__global__ void k_pick_and_advance(const float* __restrict__ best_val, const int* __restrict__ best_idx, int n,
+                                   int* __restrict__ state, int* __restrict__ history, int hist_cap) {
+    __shared__ float sv[256];
+    __shared__ int si[256];
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = best_val[i];
+        const int r = best_idx[i];
+        if (v > bv || (v == bv && r < bi)) { bv = v; bi = r; }
+    }
+    sv[threadIdx.x] = bv; si[threadIdx.x] = bi;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int t = 1; t < (int)blockDim.x; ++t)
+            if (sv[t] > bv || (sv[t] == bv && si[t] < bi)) { bv = sv[t]; bi = si[t]; }
+        const int step = state[2];
+        state[0] = bi;
+        state[1] = state[1] + 1;
+        state[2] = step + 1;
+        if (step < hist_cap) history[step] = bi;
+    }
+}
+
+__global__ void k_set_state(int* state, int token, int seq_len) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) { state[0] = token; state[1] = seq_len; state[2] = 0; }
+}
+
+__global__ void k_fill_zero(uint32_t* p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+}  // namespace
+
+// =================================================================================================
+// host side
+// =================================================================================================
+namespace {
+
+struct DeviceInfo {
+    int cus = 0;
+    bool ok = false;
+};
+
+DeviceInfo& device_info() {
+    static DeviceInfo info[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    DeviceInfo& d = info[dev];
+    if (!d.ok) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) == hipSuccess) {
+            d.cus = prop.multiProcessorCount;
+            d.ok = true;
+        }
+    }
+    return d;
+}
+
+int env_int(const char* name, int dflt) {
+    const char* v = getenv(name);
+    return v && *v ? atoi(v) : dflt;
+}
+
+constexpr size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct WorkspaceLayout {
+    size_t qkv_raw, attn_vec, inter, part_ml, part_acc, head_cnt, bar, total;
+};
+
+WorkspaceLayout workspace_layout(const cfpp_neox_dims& d) {
+    WorkspaceLayout w{};
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+    w.qkv_raw = take((size_t)3 * d.hidden * 4);
+    w.attn_vec = take((size_t)d.hidden * 2);
+    w.inter = take((size_t)d.ffn * 2);
+    w.part_ml = take((size_t)d.heads * kMaxSplit * 2 * 4);
+    w.part_acc = take((size_t)d.heads * kMaxSplit * d.head_dim * 4);
+    w.head_cnt = take((size_t)d.heads * 4);
+    w.bar = take(64);
+    w.total = off;
+    return w;
+}
+
+int check_dims(const cfpp_neox_dims* d) {
+    if (!d) return CFPP_ERR_NULL;
+    if (d->hidden <= 0 || d->heads <= 0 || d->head_dim <= 0 || d->ffn <= 0) return CFPP_ERR_DIMS;
+    if (d->hidden != d->heads * d->head_dim) return CFPP_ERR_DIMS;
+    if (d->hidden % 8 || d->ffn % 8 || d->head_dim % 8) return CFPP_ERR_DIMS;
+    if (d->head_dim > 128 || d->hidden > 8 * kChunk) return CFPP_ERR_DIMS;
+    if (d->rotary_dim < 0 || d->rotary_dim > d->head_dim || (d->rotary_dim & 1)) return CFPP_ERR_DIMS;
+    if (!(d->eps > 0.f)) return CFPP_ERR_DIMS;
+    return CFPP_OK;
+}
+
+// launch geometry for one set of dims
+struct Plan {
+    int nch;        // 512-half chunks of the hidden row (stage A registers)
+    int nwv;        // waves per workgroup
+    int ks, rg;     // stage C: K slices x row groups = nwv
+    int cpw;        // stage C chunks per wave
+};
+
+int make_plan(const cfpp_neox_dims& d, Plan* out) {
+    Plan p{};
+    p.nch = (d.hidden + kChunk - 1) / kChunk;
+    const int nchc = p.nch + (d.ffn + kChunk - 1) / kChunk;
+    if (p.nch == 5 && nchc == 25) { p.nwv = 10; p.ks = 5; p.rg = 2; p.cpw = 5; }   // Pythia-2.8B
+    else {
+        p.nwv = 8; p.ks = 8; p.rg = 1;
+        p.cpw = (nchc + p.ks - 1) / p.ks;
+    }
+    if (p.cpw > 8) return CFPP_ERR_DIMS;
+    *out = p;
+    return CFPP_OK;
+}
+
+#define CFPP_HIP(expr)                                   \
+    do {                                                 \
+        hipError_t e_ = (expr);                          \
+        if (e_ != hipSuccess) return (int)e_;            \
+    } while (0)
+
+int launch_check() {
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CFPP_OK : (int)e;
+}
+
+// ---- template dispatch ---------------------------------------------------------------------------
+template <int NCH, int NWV>
+int launch_stage_a_t(const LayerParams& p, int grid, int do_qkv, int do_up, hipStream_t st) {
+    hipLaunchKernelGGL((k_stage_a<NCH, NWV>), dim3(grid), dim3(NWV * 64), 0, st, p, do_qkv, do_up);
+    return launch_check();
+}
+template <int CPW, int NWV>
+int launch_stage_c_t(const LayerParams& p, int grid, int KS, int RG, hipStream_t st) {
+    hipLaunchKernelGGL((k_stage_c<CPW, NWV>), dim3(grid), dim3(NWV * 64), 0, st, p, KS, RG);
+    return launch_check();
+}
+template <int NCH, int CPW, int NWV>
+int launch_fused_t(const LayerParams& p, int grid, int KS, int RG, hipStream_t st) {
+    static int coop = env_int("CFPP_COOPERATIVE", 0);
+    if (coop) {
+        LayerParams pp = p;
+        void* args[] = {&pp, &KS, &RG};
+        CFPP_HIP(hipLaunchCooperativeKernel((const void*)(k_fused<NCH, CPW, NWV>), dim3(grid), dim3(NWV * 64), args, 0, st));
+        return CFPP_OK;
+    }
+    hipLaunchKernelGGL((k_fused<NCH, CPW, NWV>), dim3(grid), dim3(NWV * 64), 0, st, p, KS, RG);
+    return launch_check();
+}
+template <int NCH, int CPW, int NWV>
+int fused_max_blocks_per_cu() {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)(k_fused<NCH, CPW, NWV>), NWV * 64, 0) != hipSuccess) return 0;
+    return n;
+}
+
+#define CFPP_NCH_CASES(X) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8)
+
+int launch_stage_a(const Plan& pl, const LayerParams& p, int grid, int do_qkv, int do_up, hipStream_t st) {
+    if (pl.nwv == 10 && pl.nch == 5) return launch_stage_a_t<5, 10>(p, grid, do_qkv, do_up, st);
+    switch (pl.nch) {
+#define X(n) case n: return launch_stage_a_t<n, 8>(p, grid, do_qkv, do_up, st);
+        CFPP_NCH_CASES(X)
+#undef X
+    }
+    return CFPP_ERR_DIMS;
+}
+int launch_stage_c(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
+    if (pl.nwv == 10) return launch_stage_c_t<5, 10>(p, grid, pl.ks, pl.rg, st);
+    switch (pl.cpw) {
+#define X(n) case n: return launch_stage_c_t<n, 8>(p, grid, pl.ks, pl.rg, st);
+        CFPP_NCH_CASES(X)
+#undef X
+    }
+    return CFPP_ERR_DIMS;
+}
+// fused kernels are instantiated for the shapes that occur in the Pythia family
+#define CFPP_FUSED_CASES(X) X(1, 1, 8) X(2, 1, 8) X(2, 2, 8) X(4, 3, 8) X(5, 5, 10) X(8, 5, 8) X(8, 4, 8)
+int launch_fused(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
+#define X(a, b, c) if (pl.nch == a && pl.cpw == b && pl.nwv == c) return launch_fused_t<a, b, c>(p, grid, pl.ks, pl.rg, st);
+    CFPP_FUSED_CASES(X)
+#undef X
+    return CFPP_ERR_DIMS;
+}
+bool fused_available(const Plan& pl) {
+#define X(a, b, c) if (pl.nch == a && pl.cpw == b && pl.nwv == c) return fused_max_blocks_per_cu<a, b, c>() >= 1;
+    CFPP_FUSED_CASES(X)
+#undef X
+    return false;
+}
+
+int choose_nsplit(const cfpp_neox_dims& d, int seq_hint, int cus) {
+    // enough (head, split) items to cover the chip, at least ~64 cache rows per item
+    int by_len = (seq_hint + 63) / 64;
+    int by_chip = (cus + d.heads - 1) / d.heads;
+    int n = by_len < by_chip ? by_len : by_chip;
+    n = env_int("CFPP_NSPLIT", n);
+    if (n < 1) n = 1;
+    if (n > kMaxSplit) n = kMaxSplit;
+    return n;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_neox_io* io, void* workspace,
+                size_t ws_bytes, bool need_down, bool need_out, LayerParams* out, Plan* plan) {
+    int rc = check_dims(d);
+    if (rc) return rc;
+    if (!w || !io || !workspace) return CFPP_ERR_NULL;
+    const void* req[] = {w->ln_w, w->ln_b, w->w_qkv, w->b_qkv, w->w_o, w->b_o, w->post_ln_w, w->post_ln_b,
+                         w->w_up, w->b_up, io->input, io->k_new, io->v_new, io->k_cache, io->v_cache, io->cos, io->sin};
+    for (const void* q : req) {
+        if (!q) return CFPP_ERR_NULL;
+        if (!aligned16(q)) return CFPP_ERR_ALIGN;
+    }
+    if (need_down && (!w->w_down || !w->b_down)) return CFPP_ERR_NULL;
+    if (need_out && !io->output) return CFPP_ERR_NULL;
+    if (!need_out && (!io->attn_output || !io->mlp_intermediate)) return CFPP_ERR_NULL;
+    if (io->cache_rows < 0) return CFPP_ERR_SEQ;
+    if (!io->d_seq_len && (io->seq_len < 0 || io->seq_len > io->cache_rows)) return CFPP_ERR_SEQ;
+    const WorkspaceLayout L = workspace_layout(*d);
+    if (ws_bytes < L.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CFPP_ERR_WORKSPACE;
+    rc = make_plan(*d, plan);
+    if (rc) return rc;
+
+    LayerParams p{};
+    p.H = d->hidden; p.heads = d->heads; p.D = d->head_dim; p.rot = d->rotary_dim; p.F = d->ffn;
+    p.eps = d->eps;
+    p.qscale = (float)(1.4426950408889634 / std::sqrt((double)d->head_dim));
+    auto h = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
+    auto hm = [](void* q) { return reinterpret_cast<half_t*>(q); };
+    p.ln_w = h(w->ln_w); p.ln_b = h(w->ln_b); p.w_qkv = h(w->w_qkv); p.b_qkv = h(w->b_qkv);
+    p.w_o = h(w->w_o); p.b_o = h(w->b_o); p.ln2_w = h(w->post_ln_w); p.ln2_b = h(w->post_ln_b);
+    p.w_up = h(w->w_up); p.b_up = h(w->b_up); p.w_down = h(w->w_down); p.b_down = h(w->b_down);
+    p.x = h(io->input); p.out = hm(io->output);
+    p.k_new = hm(io->k_new); p.v_new = hm(io->v_new); p.k_cache = hm(io->k_cache); p.v_cache = hm(io->v_cache);
+    p.cache_rows = io->cache_rows;
+    p.cos = io->cos; p.sin = io->sin; p.rope_stride = io->rope_stride;
+    p.seq_len = io->seq_len; p.d_seq_len = io->d_seq_len;
+    int hint = io->d_seq_len ? (io->max_seq_len > 0 ? io->max_seq_len : io->cache_rows) : io->seq_len;
+    p.nsplit = choose_nsplit(*d, hint, device_info().cus);
+    char* ws = reinterpret_cast<char*>(workspace);
+    p.qkv_raw = reinterpret_cast<float*>(ws + L.qkv_raw);
+    p.attn_vec = reinterpret_cast<half_t*>(ws + L.attn_vec);
+    p.inter = reinterpret_cast<half_t*>(ws + L.inter);
+    p.part_ml = reinterpret_cast<float*>(ws + L.part_ml);
+    p.part_acc = reinterpret_cast<float*>(ws + L.part_acc);
+    p.head_cnt = reinterpret_cast<int*>(ws + L.head_cnt);
+    p.bar = reinterpret_cast<int*>(ws + L.bar);
+    p.c_base0 = p.x; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 1;
+    *out = p;
+    return CFPP_OK;
+}
+
+int grid_for_streaming(const Plan&) {
+    DeviceInfo& di = device_info();
+    const int cus = di.cus > 0 ? di.cus : 256;
+    return cus * env_int("CFPP_WG_PER_CU", 1);
+}
+
+int run_split(const Plan& pl, LayerParams& p, bool full_layer, hipStream_t st) {
+    const int grid = grid_for_streaming(pl);
+    int rc = launch_stage_a(pl, p, grid, 1, 1, st);
+    if (rc) return rc;
+    int bgrid = p.heads * p.nsplit;
+    hipLaunchKernelGGL(k_stage_b, dim3(bgrid), dim3(256), 0, st, p);
+    if ((rc = launch_check())) return rc;
+    (void)full_layer;
+    return launch_stage_c(pl, p, grid, st);
+}
+
+}  // namespace
+
+// =================================================================================================
+// C ABI
+// =================================================================================================
+extern "C" {
+
+const char* cfpp_version(void) { return "cfpp 0.1 (gfx950)"; }
+
+const char* cfpp_status_str(int s) {
+    switch (s) {
+        case CFPP_OK: return "ok";
+        case CFPP_ERR_NULL: return "a required pointer is NULL";
+        case CFPP_ERR_DIMS: return "unsupported layer dimensions";
+        case CFPP_ERR_SEQ: return "seq_len out of range for the KV cache";
+        case CFPP_ERR_WORKSPACE: return "workspace too small or not 256-byte aligned";
+        case CFPP_ERR_CONTEXT: return "unknown context id or pointers differ from context creation";
+        case CFPP_ERR_MODE: return "unknown mode";
+        case CFPP_ERR_DEVICE: return "device-side failure flag raised";
+        case CFPP_ERR_ALIGN: return "tensor pointer is not 16-byte aligned";
+        default: break;
+    }
+    if (s > 0) return hipGetErrorString((hipError_t)s);
+    return "unknown status";
+}
+
+size_t cfpp_neox_workspace_bytes(const cfpp_neox_dims* dims) {
+    if (check_dims(dims)) return 0;
+    return workspace_layout(*dims).total;
+}
+
+int cfpp_neox_layer_decode(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io, int mode,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+    if (mode != CFPP_MODE_FUSED && mode != CFPP_MODE_SPLIT) return CFPP_ERR_MODE;
+    LayerParams p;
+    Plan pl;
+    int rc = fill_params(dims, w, io, workspace, workspace_bytes, true, true, &p, &pl);
+    if (rc) return rc;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (mode == CFPP_MODE_SPLIT) return run_split(pl, p, true, st);
+    if (!fused_available(pl)) return CFPP_ERR_DIMS;
+    DeviceInfo& di = device_info();
+    const int grid = di.cus > 0 ? di.cus : 256;
+    return launch_fused(pl, p, grid, st);
+}
+
+int cfpp_neox_attention_mlp_up(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+    LayerParams p;
+    Plan pl;
+    int rc = fill_params(dims, w, io, workspace, workspace_bytes, false, false, &p, &pl);
+    if (rc) return rc;
+    if (!aligned16(io->attn_output) || !aligned16(io->mlp_intermediate)) return CFPP_ERR_ALIGN;
+    p.inter = reinterpret_cast<half_t*>(io->mlp_intermediate);   // MLP-up writes the caller's tensor directly
+    p.out = reinterpret_cast<half_t*>(io->attn_output);          // stage C: W_o attn + b_o only
+    p.c_base0 = nullptr; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 0;
+    return run_split(pl, p, false, reinterpret_cast<hipStream_t>(stream));
+}
+
+int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void* attn_output,
+                       const void* mlp_intermediate, const void* w_down, const void* b_down, void* output,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_dims(dims);
+    if (rc) return rc;
+    const void* req[] = {input, attn_output, mlp_intermediate, w_down, b_down, output};
+    for (const void* q : req) {
+        if (!q) return CFPP_ERR_NULL;
+        if (!aligned16(q)) return CFPP_ERR_ALIGN;
+    }
+    (void)workspace; (void)workspace_bytes;
+    Plan pl;
+    if ((rc = make_plan(*dims, &pl))) return rc;
+    LayerParams p{};
+    p.H = dims->hidden; p.heads = dims->heads; p.D = dims->head_dim; p.rot = dims->rotary_dim; p.F = dims->ffn;
+    p.w_down = reinterpret_cast<const half_t*>(w_down); p.b_down = reinterpret_cast<const half_t*>(b_down);
+    p.inter = const_cast<half_t*>(reinterpret_cast<const half_t*>(mlp_intermediate));
+    p.out = reinterpret_cast<half_t*>(output);
+    p.c_base0 = reinterpret_cast<const half_t*>(input);
+    p.c_base1 = reinterpret_cast<const half_t*>(attn_output);
+    p.c_use_o = 0; p.c_use_down = 1;
+    return launch_stage_c(pl, p, grid_for_streaming(pl), reinterpret_cast<hipStream_t>(stream));
+}
+
+int cfpp_workspace_check(const cfpp_neox_dims* dims, void* workspace, void* stream) {
+    if (check_dims(dims)) return CFPP_ERR_DIMS;
+    if (!workspace) return CFPP_ERR_NULL;
+    const WorkspaceLayout L = workspace_layout(*dims);
+    int* bar = reinterpret_cast<int*>(reinterpret_cast<char*>(workspace) + L.bar);
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    int host[3] = {0, 0, 0};
+    CFPP_HIP(hipMemcpyAsync(host, bar, sizeof(host), hipMemcpyDeviceToHost, st));
+    CFPP_HIP(hipStreamSynchronize(st));
+    if (host[2] != 0 || host[0] != 0 || host[1] != 0) {
+        // a raised flag (or counters left mid-flight by an expired wait): clear so the workspace is reusable
+        CFPP_HIP(hipMemsetAsync(workspace, 0, L.total, st));
+        CFPP_HIP(hipStreamSynchronize(st));
+        return CFPP_ERR_DEVICE;
+    }
+    return CFPP_OK;
+}
+
+// ---- per-layer contexts --------------------------------------------------------------------------
+namespace {
+struct Ctx {
+    cfpp_neox_dims dims{};
+    const void *w_qkv = nullptr, *w_o = nullptr, *w_up = nullptr, *w_down = nullptr;
+    void *k_cache = nullptr, *v_cache = nullptr;
+    int cache_rows = 0, max_seq_len = 0, device = 0;
+    void* slab = nullptr;          // output | k_new | v_new | workspace
+    cfpp_ctx_buffers bufs{};
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+};
+std::map<std::pair<int, int64_t>, Ctx> g_ctx;
+std::mutex g_ctx_mu;
+
+void ctx_release(Ctx& c) {
+    if (c.slab) {
+        int cur = 0;
+        (void)hipGetDevice(&cur);
+        if (cur != c.device) (void)hipSetDevice(c.device);
+        (void)hipFree(c.slab);
+        if (cur != c.device) (void)hipSetDevice(cur);
+        c.slab = nullptr;
+    }
+}
+}  // namespace
+
+int cfpp_ctx_create(int family, int64_t id, const cfpp_neox_dims* dims, const void* w_qkv, const void* w_o,
+                    const void* w_up, const void* w_down, void* k_cache, void* v_cache, int32_t cache_rows,
+                    int32_t max_seq_len, cfpp_ctx_buffers* out_buffers) {
+    int rc = check_dims(dims);
+    if (rc) return rc;
+    Plan pl;
+    if ((rc = make_plan(*dims, &pl))) return rc;
+    if (!w_qkv || !w_o || !w_up || !w_down || !k_cache || !v_cache) return CFPP_ERR_NULL;
+    if (cache_rows <= 0 || max_seq_len < 0 || max_seq_len > cache_rows) return CFPP_ERR_SEQ;
+    Ctx c;
+    c.dims = *dims;
+    c.w_qkv = w_qkv; c.w_o = w_o; c.w_up = w_up; c.w_down = w_down;
+    c.k_cache = k_cache; c.v_cache = v_cache; c.cache_rows = cache_rows;
+    c.max_seq_len = max_seq_len > 0 ? max_seq_len : cache_rows;
+    CFPP_HIP(hipGetDevice(&c.device));
+    const size_t hb = align_up((size_t)dims->hidden * 2, 256);
+    c.ws_bytes = workspace_layout(*dims).total;
+    CFPP_HIP(hipMalloc(&c.slab, 3 * hb + c.ws_bytes));
+    hipError_t e = hipMemset(c.slab, 0, 3 * hb + c.ws_bytes);
+    if (e != hipSuccess) { (void)hipFree(c.slab); return (int)e; }
+    char* base = reinterpret_cast<char*>(c.slab);
+    c.bufs.output = base; c.bufs.k_new = base + hb; c.bufs.v_new = base + 2 * hb;
+    c.ws = base + 3 * hb;
+    std::lock_guard<std::mutex> lock(g_ctx_mu);
+    auto key = std::make_pair(family, id);
+    auto it = g_ctx.find(key);
+    if (it != g_ctx.end()) { ctx_release(it->second); g_ctx.erase(it); }
+    g_ctx[key] = c;
+    if (out_buffers) *out_buffers = c.bufs;
+    return CFPP_OK;
+}
+
+int cfpp_ctx_step(int family, int64_t id, const cfpp_neox_weights* w, const cfpp_neox_io* io, int mode, void* stream,
+                  cfpp_ctx_buffers* out_buffers) {
+    if (!w || !io) return CFPP_ERR_NULL;
+    Ctx c;
+    {
+        std::lock_guard<std::mutex> lock(g_ctx_mu);
+        auto it = g_ctx.find(std::make_pair(family, id));
+        if (it == g_ctx.end()) return CFPP_ERR_CONTEXT;
+        c = it->second;
+    }
+    if (io->k_cache != c.k_cache || io->v_cache != c.v_cache) return CFPP_ERR_CONTEXT;
+    if ((w->w_qkv && w->w_qkv != c.w_qkv) || (w->w_o && w->w_o != c.w_o) || (w->w_up && w->w_up != c.w_up) ||
+        (w->w_down && w->w_down != c.w_down))
+        return CFPP_ERR_CONTEXT;
+    cfpp_neox_weights ww = *w;
+    ww.w_qkv = c.w_qkv; ww.w_o = c.w_o; ww.w_up = c.w_up; ww.w_down = c.w_down;
+    cfpp_neox_io ii = *io;
+    ii.output = c.bufs.output; ii.k_new = c.bufs.k_new; ii.v_new = c.bufs.v_new;
+    ii.cache_rows = c.cache_rows;
+    if (ii.max_seq_len <= 0) ii.max_seq_len = c.max_seq_len;
+    if (out_buffers) *out_buffers = c.bufs;
+    return cfpp_neox_layer_decode(&c.dims, &ww, &ii, mode, c.ws, c.ws_bytes, stream);
+}
+
+int cfpp_ctx_destroy(int family, int64_t id) {
+    std::lock_guard<std::mutex> lock(g_ctx_mu);
+    auto it = g_ctx.find(std::make_pair(family, id));
+    if (it == g_ctx.end()) return CFPP_OK;
+    ctx_release(it->second);
+    g_ctx.erase(it);
+    return CFPP_OK;
+}
+
+// ---- LM head -------------------------------------------------------------------------------------
+namespace {
+int launch_lm_head(int H, int vocab, float eps, const void* x, const void* ln_w, const void* ln_b, const void* W,
+                   float* logits, float* best_val, int* best_idx, int grid, hipStream_t st) {
+    const int nch = (H + kChunk - 1) / kChunk;
+    auto h = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
+    switch (nch) {
+#define X(n)                                                                                                    \
+    case n:                                                                                                     \
+        hipLaunchKernelGGL((k_lm_head<n, 8>), dim3(grid), dim3(512), 0, st, h(x), H, eps, h(ln_w), h(ln_b), h(W), \
+                           vocab, logits, best_val, best_idx);                                                  \
+        return launch_check();
+        CFPP_NCH_CASES(X)
+#undef X
+    }
+    return CFPP_ERR_DIMS;
+}
+}  // namespace
+
+int cfpp_neox_lm_head(int32_t hidden, int32_t vocab, float eps, const void* x, const void* ln_w, const void* ln_b,
+                      const void* w, float* logits, void* stream) {
+    if (!x || !ln_w || !ln_b || !w || !logits) return CFPP_ERR_NULL;
+    if (hidden <= 0 || hidden % 8 || hidden > 8 * kChunk || vocab <= 0) return CFPP_ERR_DIMS;
+    if (!aligned16(x) || !aligned16(ln_w) || !aligned16(ln_b) || !aligned16(w)) return CFPP_ERR_ALIGN;
+    Plan pl{};
+    return launch_lm_head(hidden, vocab, eps, x, ln_w, ln_b, w, logits, nullptr, nullptr, grid_for_streaming(pl),
+                          reinterpret_cast<hipStream_t>(stream));
+}
+
+// ---- whole-model decode --------------------------------------------------------------------------
+struct cfpp_neox_stack {
+    cfpp_neox_stack_desc desc{};
+    std::vector<cfpp_neox_weights> layers;
+    std::vector<void*> kc, vc;
+    Plan plan{};
+    int device = 0, grid = 0;
+    char* slab = nullptr;
+    int* state = nullptr;         // {token, seq_len, step}
+    half_t* hidden[2] = {nullptr, nullptr};
+    half_t *k_new = nullptr, *v_new = nullptr;
+    float* logits = nullptr;
+    float* best_val = nullptr;
+    int* best_idx = nullptr;
+    int* history = nullptr;
+    int hist_cap = 0;
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+    hipStream_t own_stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipStream_t exec_stream = nullptr;
+};
+
+namespace {
+int stack_enqueue_step(cfpp_neox_stack* s, hipStream_t st) {
+    const cfpp_neox_dims& d = s->desc.dims;
+    const int H = d.hidden;
+    hipLaunchKernelGGL(k_embed, dim3((H / 8 + 255) / 256), dim3(256), 0, st,
+                       reinterpret_cast<const half_t*>(s->desc.embed), s->state, H, s->desc.vocab, s->hidden[0]);
+    int rc = launch_check();
+    if (rc) return rc;
+    for (int l = 0; l < s->desc.n_layers; ++l) {
+        cfpp_neox_io io{};
+        io.input = s->hidden[l & 1];
+        io.output = s->hidden[(l + 1) & 1];
+        io.k_new = s->k_new; io.v_new = s->v_new;
+        io.k_cache = s->kc[l]; io.v_cache = s->vc[l];
+        io.cache_rows = s->desc.cache_rows;
+        io.cos = s->desc.rope_cos; io.sin = s->desc.rope_sin;
+        io.rope_stride = d.rotary_dim;
+        io.seq_len = 0;
+        io.d_seq_len = s->state + 1;
+        io.max_seq_len = s->desc.cache_rows;
+        rc = cfpp_neox_layer_decode(&d, &s->layers[l], &io, s->desc.mode, s->ws, s->ws_bytes, st);
+        if (rc) return rc;
+    }
+    rc = launch_lm_head(H, s->desc.vocab, d.eps, s->hidden[s->desc.n_layers & 1], s->desc.final_ln_w, s->desc.final_ln_b,
+                        s->desc.lm_head, s->logits, s->best_val, s->best_idx, s->grid, st);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_pick_and_advance, dim3(1), dim3(256), 0, st, s->best_val, s->best_idx, s->grid, s->state,
+                       s->history, s->hist_cap);
+    return launch_check();
+}
+}  // namespace
+
+int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out) {
+    if (!desc || !out) return CFPP_ERR_NULL;
+    int rc = check_dims(&desc->dims);
+    if (rc) return rc;
+    if (desc->n_layers <= 0 || desc->vocab <= 0 || desc->cache_rows <= 0) return CFPP_ERR_DIMS;
+    if (!desc->layers || !desc->embed || !desc->final_ln_w || !desc->final_ln_b || !desc->lm_head || !desc->k_caches ||
+        !desc->v_caches || !desc->rope_cos || !desc->rope_sin)
+        return CFPP_ERR_NULL;
+    if (desc->mode != CFPP_MODE_FUSED && desc->mode != CFPP_MODE_SPLIT) return CFPP_ERR_MODE;
+    cfpp_neox_stack* s = new cfpp_neox_stack();
+    s->desc = *desc;
+    s->layers.assign(desc->layers, desc->layers + desc->n_layers);
+    s->kc.assign(desc->k_caches, desc->k_caches + desc->n_layers);
+    s->vc.assign(desc->v_caches, desc->v_caches + desc->n_layers);
+    s->desc.layers = nullptr; s->desc.k_caches = nullptr; s->desc.v_caches = nullptr;
+    if ((rc = make_plan(desc->dims, &s->plan))) { delete s; return rc; }
+    hipError_t e = hipGetDevice(&s->device);
+    if (e != hipSuccess) { delete s; return (int)e; }
+    s->grid = grid_for_streaming(s->plan);
+    s->hist_cap = 1 << 16;
+    const cfpp_neox_dims& d = desc->dims;
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+    const size_t o_state = take(64), o_h0 = take((size_t)d.hidden * 2), o_h1 = take((size_t)d.hidden * 2);
+    const size_t o_k = take((size_t)d.hidden * 2), o_v = take((size_t)d.hidden * 2);
+    const size_t o_logits = take((size_t)desc->vocab * 4);
+    const size_t o_bv = take((size_t)s->grid * 4), o_bi = take((size_t)s->grid * 4);
+    const size_t o_hist = take((size_t)s->hist_cap * 4);
+    s->ws_bytes = workspace_layout(d).total;
+    const size_t o_ws = take(s->ws_bytes);
+    e = hipMalloc(reinterpret_cast<void**>(&s->slab), off);
+    if (e != hipSuccess) { delete s; return (int)e; }
+    e = hipMemset(s->slab, 0, off);
+    if (e != hipSuccess) { (void)hipFree(s->slab); delete s; return (int)e; }
+    s->state = reinterpret_cast<int*>(s->slab + o_state);
+    s->hidden[0] = reinterpret_cast<half_t*>(s->slab + o_h0);
+    s->hidden[1] = reinterpret_cast<half_t*>(s->slab + o_h1);
+    s->k_new = reinterpret_cast<half_t*>(s->slab + o_k);
+    s->v_new = reinterpret_cast<half_t*>(s->slab + o_v);
+    s->logits = reinterpret_cast<float*>(s->slab + o_logits);
+    s->best_val = reinterpret_cast<float*>(s->slab + o_bv);
+    s->best_idx = reinterpret_cast<int*>(s->slab + o_bi);
+    s->history = reinterpret_cast<int*>(s->slab + o_hist);
+    s->ws = s->slab + o_ws;
+    *out = s;
+    return CFPP_OK;
+}
+
+int cfpp_stack_set_state(cfpp_neox_stack* s, int32_t token, int32_t seq_len, void* stream) {
+    if (!s) return CFPP_ERR_NULL;
+    if (seq_len < 0 || seq_len > s->desc.cache_rows) return CFPP_ERR_SEQ;
+    if (token < 0 || token >= s->desc.vocab) return CFPP_ERR_DIMS;
+    hipLaunchKernelGGL(k_set_state, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(stream), s->state, token, seq_len);
+    return launch_check();
+}
+
+int cfpp_stack_step(cfpp_neox_stack* s, void* stream) {
+    if (!s) return CFPP_ERR_NULL;
+    return stack_enqueue_step(s, reinterpret_cast<hipStream_t>(stream));
+}
+
+int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream) {
+    if (!s) return CFPP_ERR_NULL;
+    if (n_steps < 0) return CFPP_ERR_DIMS;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (!st) {
+        if (!s->own_stream) CFPP_HIP(hipStreamCreateWithFlags(&s->own_stream, hipStreamNonBlocking));
+        st = s->own_stream;
+    }
+    if (!s->exec) {
+        CFPP_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeRelaxed));
+        int rc = stack_enqueue_step(s, st);
+        hipGraph_t g = nullptr;
+        hipError_t e = hipStreamEndCapture(st, &g);
+        if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
+        if (e != hipSuccess) return (int)e;
+        s->graph = g;
+        CFPP_HIP(hipGraphInstantiate(&s->exec, s->graph, nullptr, nullptr, 0));
+    }
+    for (int i = 0; i < n_steps; ++i) CFPP_HIP(hipGraphLaunch(s->exec, st));
+    if (!stream) CFPP_HIP(hipStreamSynchronize(st));
+    return CFPP_OK;
+}
+
+int cfpp_stack_buffers(cfpp_neox_stack* s, float** logits, void** hidden, int32_t** state, int32_t** history,
+                       int32_t* history_capacity) {
+    if (!s) return CFPP_ERR_NULL;
+    if (logits) *logits = s->logits;
+    if (hidden) *hidden = s->hidden[s->desc.n_layers & 1];
+    if (state) *state = s->state;
+    if (history) *history = s->history;
+    if (history_capacity) *history_capacity = s->hist_cap;
+    return CFPP_OK;
+}
+
+int cfpp_stack_destroy(cfpp_neox_stack* s) {
+    if (!s) return CFPP_OK;
+    if (s->exec) (void)hipGraphExecDestroy(s->exec);
+    if (s->graph) (void)hipGraphDestroy(s->graph);
+    if (s->own_stream) (void)hipStreamDestroy(s->own_stream);
+    if (s->slab) (void)hipFree(s->slab);
+    delete s;
+    return CFPP_OK;
+}
+
+}  // extern "C"

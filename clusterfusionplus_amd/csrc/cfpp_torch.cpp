@@ -1,0 +1,463 @@
+// PyTorch-ROCm binding: the `clusterfusion` Python operator surface on top of the C ABI (cfpp.h).
+//
+// Same Python names, positional argument order and return tuples as the reference's binding table
+// (reference include/pybind.cpp:280-297); the reference's C++ forward declarations that fix the
+// argument meaning are include/pybind.cpp:109-267.  Differences, all on the safe side:
+//   * every tensor is validated (device, dtype, contiguity, element count, cache capacity) and a bad
+//     argument raises RuntimeError instead of reading out of bounds (the reference checks nothing);
+//   * launches go to torch's current HIP stream without device-wide synchronisation;
+//   * a cache with exactly `current_seq_len` rows is accepted: the append is skipped, k/v are returned;
+//   * `graph_decode_step` also accepts a device int32 tensor as `current_seq_len` (with cos/sin given
+//     as `[positions, rotary_dim]` tables), which makes the step replayable from a captured HIP graph.
+// This file contains no device code; torch is used for tensors, streams and exceptions only.
+#include <torch/extension.h>
+#include <c10/hip/HIPStream.h>
+#include <c10/hip/HIPGuard.h>
+
+#include <map>
+#include <memory>
+#include <mutex>
+#include <tuple>
+#include <vector>
+
+#include "cfpp.h"
+
+namespace {
+
+using torch::Tensor;
+
+struct Model {
+    const char* name;
+    int family;
+    cfpp_neox_dims dims;
+};
+const Model kPythia2b8{"pythia_2b8", 0, {2560, 32, 80, 20, 10240, 1e-5f}};
+const Model kPythia6b9{"pythia_6b9", 1, {4096, 32, 128, 32, 16384, 1e-5f}};
+
+void check_rc(int rc, const char* what) {
+    TORCH_CHECK(rc == 0, what, ": ", cfpp_status_str(rc), " (status ", rc, ")");
+}
+
+void check_half(const Tensor& t, const char* name, int64_t numel, const Tensor& like) {
+    TORCH_CHECK(t.defined(), name, " is undefined");
+    TORCH_CHECK(t.is_cuda(), name, " must be a GPU tensor");
+    TORCH_CHECK(t.device() == like.device(), name, " is on ", t.device(), " but input is on ", like.device());
+    TORCH_CHECK(t.scalar_type() == torch::kFloat16, name, " must be float16, got ", t.scalar_type());
+    TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+    TORCH_CHECK(t.numel() == numel, name, " must have ", numel, " elements, got ", t.numel());
+}
+
+void check_rope(const Tensor& t, const char* name, int64_t min_numel, const Tensor& like) {
+    TORCH_CHECK(t.defined() && t.is_cuda() && t.device() == like.device(), name, " must be a GPU tensor on the input's device");
+    TORCH_CHECK(t.scalar_type() == torch::kFloat32, name, " must be float32, got ", t.scalar_type());
+    TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+    TORCH_CHECK(t.numel() >= min_numel, name, " must have at least ", min_numel, " elements, got ", t.numel());
+}
+
+int64_t check_cache(const Tensor& t, const char* name, int64_t H, const Tensor& like) {
+    TORCH_CHECK(t.defined() && t.is_cuda() && t.device() == like.device(), name, " must be a GPU tensor on the input's device");
+    TORCH_CHECK(t.scalar_type() == torch::kFloat16, name, " must be float16");
+    TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+    TORCH_CHECK(t.dim() == 2 && t.size(1) == H, name, " must have shape [rows, ", H, "]");
+    return t.size(0);
+}
+
+// one zero-initialised scratch buffer per (device, stream): calls on one stream are ordered, so they can share
+Tensor workspace_for(const cfpp_neox_dims& d, const torch::Device& dev, hipStream_t st) {
+    static std::mutex mu;
+    static std::map<std::tuple<int, void*, int, int>, Tensor> cache;
+    std::lock_guard<std::mutex> lock(mu);
+    auto key = std::make_tuple((int)dev.index(), (void*)st, (int)d.hidden, (int)d.ffn);
+    auto it = cache.find(key);
+    if (it != cache.end()) return it->second;
+    const int64_t bytes = (int64_t)cfpp_neox_workspace_bytes(&d);
+    TORCH_CHECK(bytes > 0, "unsupported layer dimensions");
+    Tensor ws = torch::zeros({bytes + 256}, torch::TensorOptions().dtype(torch::kUInt8).device(dev));
+    cache[key] = ws;
+    return ws;
+}
+void* ws_ptr(const Tensor& ws) {
+    auto p = reinterpret_cast<uintptr_t>(ws.data_ptr());
+    return reinterpret_cast<void*>((p + 255) / 256 * 256);
+}
+
+struct LayerArgs {
+    Tensor input, weight_qkv, bias_qkv, weight_o, bias_o, k_cache, v_cache, ln_w, ln_b, cos, sin, post_ln_w,
+        post_ln_b, up_w, up_b, down_w, down_b;
+};
+
+void fill_weights(const cfpp_neox_dims& d, const LayerArgs& a, bool need_down, cfpp_neox_weights* w) {
+    const int64_t H = d.hidden, F = d.ffn;
+    check_half(a.input, "input", H, a.input);
+    check_half(a.weight_qkv, "weight_qkv", 3 * H * H, a.input);
+    check_half(a.bias_qkv, "bias_qkv", 3 * H, a.input);
+    check_half(a.weight_o, "weight_o", H * H, a.input);
+    check_half(a.bias_o, "bias_o", H, a.input);
+    check_half(a.ln_w, "layernorm_weight", H, a.input);
+    check_half(a.ln_b, "layernorm_bias", H, a.input);
+    check_half(a.post_ln_w, "post_ln_weight", H, a.input);
+    check_half(a.post_ln_b, "post_ln_bias", H, a.input);
+    check_half(a.up_w, "mlp_up_weight", F * H, a.input);
+    check_half(a.up_b, "mlp_up_bias", F, a.input);
+    if (need_down) {
+        check_half(a.down_w, "mlp_down_weight", H * F, a.input);
+        check_half(a.down_b, "mlp_down_bias", H, a.input);
+    }
+    w->ln_w = a.ln_w.data_ptr(); w->ln_b = a.ln_b.data_ptr();
+    w->w_qkv = a.weight_qkv.data_ptr(); w->b_qkv = a.bias_qkv.data_ptr();
+    w->w_o = a.weight_o.data_ptr(); w->b_o = a.bias_o.data_ptr();
+    w->post_ln_w = a.post_ln_w.data_ptr(); w->post_ln_b = a.post_ln_b.data_ptr();
+    w->w_up = a.up_w.data_ptr(); w->b_up = a.up_b.data_ptr();
+    w->w_down = need_down ? a.down_w.data_ptr() : nullptr;
+    w->b_down = need_down ? a.down_b.data_ptr() : nullptr;
+}
+
+void fill_io(const cfpp_neox_dims& d, const LayerArgs& a, int64_t seq_len, cfpp_neox_io* io) {
+    const int64_t H = d.hidden;
+    const int64_t rows_k = check_cache(a.k_cache, "k_cache", H, a.input);
+    const int64_t rows_v = check_cache(a.v_cache, "v_cache", H, a.input);
+    TORCH_CHECK(seq_len >= 0, "current_seq_len must be >= 0, got ", seq_len);
+    TORCH_CHECK(rows_k >= seq_len && rows_v >= seq_len, "current_seq_len ", seq_len, " exceeds the cache rows (k ",
+                rows_k, ", v ", rows_v, ")");
+    check_rope(a.cos, "cos", d.rotary_dim, a.input);
+    check_rope(a.sin, "sin", d.rotary_dim, a.input);
+    *io = cfpp_neox_io{};
+    io->input = a.input.data_ptr();
+    io->k_cache = a.k_cache.data_ptr(); io->v_cache = a.v_cache.data_ptr();
+    io->cache_rows = (int32_t)std::min(rows_k, rows_v);
+    io->cos = a.cos.data_ptr<float>(); io->sin = a.sin.data_ptr<float>();
+    io->rope_stride = 0;
+    io->seq_len = (int32_t)seq_len;
+}
+
+std::tuple<Tensor, Tensor, Tensor> decoder_layer(const Model& m, int mode, const LayerArgs& a, int64_t seq_len) {
+    const cfpp_neox_dims& d = m.dims;
+    cfpp_neox_weights w;
+    cfpp_neox_io io;
+    fill_weights(d, a, true, &w);
+    fill_io(d, a, seq_len, &io);
+    c10::hip::HIPGuard guard(a.input.device());
+    auto opts = a.input.options();
+    Tensor out = torch::empty({1, d.hidden}, opts);
+    Tensor k = torch::empty({1, d.heads, d.head_dim}, opts);
+    Tensor v = torch::empty({1, d.heads, d.head_dim}, opts);
+    io.output = out.data_ptr(); io.k_new = k.data_ptr(); io.v_new = v.data_ptr();
+    hipStream_t st = c10::hip::getCurrentHIPStream().stream();
+    Tensor ws = workspace_for(d, a.input.device(), st);
+    check_rc(cfpp_neox_layer_decode(&d, &w, &io, mode, ws_ptr(ws), cfpp_neox_workspace_bytes(&d), st), m.name);
+    return std::make_tuple(out, k, v);
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> attention_only(const Model& m, const LayerArgs& a, int64_t seq_len) {
+    const cfpp_neox_dims& d = m.dims;
+    cfpp_neox_weights w;
+    cfpp_neox_io io;
+    fill_weights(d, a, false, &w);
+    fill_io(d, a, seq_len, &io);
+    c10::hip::HIPGuard guard(a.input.device());
+    auto opts = a.input.options();
+    Tensor attn = torch::empty({1, d.hidden}, opts);
+    Tensor inter = torch::empty({d.ffn}, opts);
+    Tensor k = torch::empty({1, d.heads, d.head_dim}, opts);
+    Tensor v = torch::empty({1, d.heads, d.head_dim}, opts);
+    io.attn_output = attn.data_ptr(); io.mlp_intermediate = inter.data_ptr();
+    io.k_new = k.data_ptr(); io.v_new = v.data_ptr();
+    hipStream_t st = c10::hip::getCurrentHIPStream().stream();
+    Tensor ws = workspace_for(d, a.input.device(), st);
+    check_rc(cfpp_neox_attention_mlp_up(&d, &w, &io, ws_ptr(ws), cfpp_neox_workspace_bytes(&d), st), m.name);
+    return std::make_tuple(attn, inter, k, v);
+}
+
+Tensor mlp_only(const Model& m, Tensor input, Tensor attn_output, Tensor inter, Tensor down_w, Tensor down_b) {
+    const cfpp_neox_dims& d = m.dims;
+    check_half(input, "input", d.hidden, input);
+    check_half(attn_output, "attn_output", d.hidden, input);
+    check_half(inter, "mlp_intermediate", d.ffn, input);
+    check_half(down_w, "mlp_down_weight", (int64_t)d.hidden * d.ffn, input);
+    check_half(down_b, "mlp_down_bias", d.hidden, input);
+    c10::hip::HIPGuard guard(input.device());
+    Tensor out = torch::empty({1, d.hidden}, input.options());
+    hipStream_t st = c10::hip::getCurrentHIPStream().stream();
+    check_rc(cfpp_neox_mlp_down(&d, input.data_ptr(), attn_output.data_ptr(), inter.data_ptr(), down_w.data_ptr(),
+                                down_b.data_ptr(), out.data_ptr(), nullptr, 0, st), m.name);
+    return out;
+}
+
+// ---- decode contexts -----------------------------------------------------------------------------
+struct PyCtx {
+    Tensor k_cache, v_cache, w_qkv, w_o, w_up, w_down;   // keep the storage alive (the reference keeps raw pointers)
+    Tensor output, k_new, v_new;                          // views of the context-owned device buffers
+};
+std::mutex g_mu;
+std::map<std::pair<int, int64_t>, PyCtx> g_ctx;
+
+void create_graph_context(const Model& m, int64_t id, Tensor k_cache, Tensor v_cache, Tensor w_qkv, Tensor w_o,
+                          Tensor w_up, Tensor w_down, int64_t max_seq_len) {
+    const cfpp_neox_dims& d = m.dims;
+    const int64_t H = d.hidden, F = d.ffn;
+    const int64_t rows_k = check_cache(k_cache, "k_cache", H, k_cache);
+    const int64_t rows_v = check_cache(v_cache, "v_cache", H, k_cache);
+    check_half(w_qkv, "weight_qkv", 3 * H * H, k_cache);
+    check_half(w_o, "weight_o", H * H, k_cache);
+    check_half(w_up, "mlp_up_weight", F * H, k_cache);
+    check_half(w_down, "mlp_down_weight", H * F, k_cache);
+    const int64_t rows = std::min(rows_k, rows_v);
+    TORCH_CHECK(max_seq_len > 0 && max_seq_len <= rows, "max_seq_len ", max_seq_len, " must be in [1, cache rows = ", rows, "]");
+    c10::hip::HIPGuard guard(k_cache.device());
+    cfpp_ctx_buffers b{};
+    check_rc(cfpp_ctx_create(m.family, id, &d, w_qkv.data_ptr(), w_o.data_ptr(), w_up.data_ptr(), w_down.data_ptr(),
+                             k_cache.data_ptr(), v_cache.data_ptr(), (int32_t)rows, (int32_t)max_seq_len, &b),
+             "create_graph_context");
+    auto opts = k_cache.options();
+    PyCtx c{k_cache, v_cache, w_qkv, w_o, w_up, w_down,
+            torch::from_blob(b.output, {1, H}, opts),
+            torch::from_blob(b.k_new, {1, (int64_t)d.heads, (int64_t)d.head_dim}, opts),
+            torch::from_blob(b.v_new, {1, (int64_t)d.heads, (int64_t)d.head_dim}, opts)};
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_ctx[std::make_pair(m.family, id)] = c;
+}
+
+std::tuple<Tensor, Tensor, Tensor> graph_decode_step(const Model& m, int64_t id, Tensor input, Tensor ln_w, Tensor ln_b,
+                                                     Tensor qkv_bias, Tensor o_bias, Tensor cos, Tensor sin, Tensor k_cache,
+                                                     Tensor v_cache, Tensor post_ln_w, Tensor post_ln_b, Tensor up_b,
+                                                     Tensor down_b, py::object current_seq_len) {
+    const cfpp_neox_dims& d = m.dims;
+    PyCtx c;
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        auto it = g_ctx.find(std::make_pair(m.family, id));
+        // the reference raises std::runtime_error("Graph context not initialized...") here
+        // (include/5090/pythia_2b8/pythia_kernel_dispatch_graph.cu:231-233)
+        TORCH_CHECK(it != g_ctx.end(), "Graph context ", id, " not initialized: call ", m.name, "_create_graph_context first");
+        c = it->second;
+    }
+    const int64_t H = d.hidden, F = d.ffn;
+    check_half(input, "input", H, input);
+    check_half(ln_w, "layernorm_weight", H, input);
+    check_half(ln_b, "layernorm_bias", H, input);
+    check_half(qkv_bias, "qkv_bias", 3 * H, input);
+    check_half(o_bias, "o_bias", H, input);
+    check_half(post_ln_w, "post_ln_weight", H, input);
+    check_half(post_ln_b, "post_ln_bias", H, input);
+    check_half(up_b, "mlp_up_bias", F, input);
+    check_half(down_b, "mlp_down_bias", H, input);
+    TORCH_CHECK(k_cache.data_ptr() == c.k_cache.data_ptr() && v_cache.data_ptr() == c.v_cache.data_ptr(),
+                "k_cache / v_cache differ from the tensors the context was created with");
+    check_rope(cos, "cos", d.rotary_dim, input);
+    check_rope(sin, "sin", d.rotary_dim, input);
+
+    cfpp_neox_weights w{};
+    w.ln_w = ln_w.data_ptr(); w.ln_b = ln_b.data_ptr(); w.b_qkv = qkv_bias.data_ptr(); w.b_o = o_bias.data_ptr();
+    w.post_ln_w = post_ln_w.data_ptr(); w.post_ln_b = post_ln_b.data_ptr(); w.b_up = up_b.data_ptr(); w.b_down = down_b.data_ptr();
+    cfpp_neox_io io{};
+    io.input = input.data_ptr();
+    io.k_cache = k_cache.data_ptr(); io.v_cache = v_cache.data_ptr();
+    io.cos = cos.data_ptr<float>(); io.sin = sin.data_ptr<float>();
+    const int64_t rows = std::min(c.k_cache.size(0), c.v_cache.size(0));
+    Tensor seq_t;
+    if (THPVariable_Check(current_seq_len.ptr())) {
+        seq_t = THPVariable_Unpack(current_seq_len.ptr());
+        TORCH_CHECK(seq_t.is_cuda() && seq_t.device() == input.device() && seq_t.scalar_type() == torch::kInt32 && seq_t.numel() == 1,
+                    "a tensor current_seq_len must be one int32 on the input's device");
+        TORCH_CHECK(cos.dim() == 2 && sin.dim() == 2 && cos.size(1) >= d.rotary_dim && cos.sizes() == sin.sizes() &&
+                        cos.size(0) >= rows,
+                    "with a tensor current_seq_len, cos/sin must be [positions >= cache rows, >= rotary_dim] tables");
+        io.d_seq_len = seq_t.data_ptr<int32_t>();
+        io.rope_stride = (int32_t)cos.size(1);
+    } else {
+        const int64_t s = current_seq_len.cast<int64_t>();
+        TORCH_CHECK(s >= 0 && s <= rows, "current_seq_len ", s, " out of range for ", rows, " cache rows");
+        io.seq_len = (int32_t)s;
+    }
+    c10::hip::HIPGuard guard(input.device());
+    hipStream_t st = c10::hip::getCurrentHIPStream().stream();
+    check_rc(cfpp_ctx_step(m.family, id, &w, &io, CFPP_MODE_FUSED, st, nullptr), "graph_decode_step");
+    return std::make_tuple(c.output, c.k_new, c.v_new);
+}
+
+void destroy_graph_context(const Model& m, int64_t id) {
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        g_ctx.erase(std::make_pair(m.family, id));
+    }
+    check_rc(cfpp_ctx_destroy(m.family, id), "destroy_graph_context");
+}
+
+// ---- whole-model decode (our counterpart of the reference's Python decode loop) --------------------
+struct PyStack {
+    cfpp_neox_stack* s = nullptr;
+    std::vector<Tensor> keep;
+    cfpp_neox_dims dims{};
+    int64_t vocab = 0;
+    torch::Device device{torch::kCPU};
+    ~PyStack() { if (s) cfpp_stack_destroy(s); }
+};
+
+std::shared_ptr<PyStack> stack_create(int64_t hidden, int64_t heads, int64_t head_dim, int64_t rotary_dim, int64_t ffn,
+                                      double eps, std::vector<std::vector<Tensor>> layers, Tensor embed, Tensor final_ln_w,
+                                      Tensor final_ln_b, Tensor lm_head, std::vector<Tensor> k_caches,
+                                      std::vector<Tensor> v_caches, Tensor rope_cos, Tensor rope_sin, int64_t mode) {
+    auto ps = std::make_shared<PyStack>();
+    cfpp_neox_dims d{(int32_t)hidden, (int32_t)heads, (int32_t)head_dim, (int32_t)rotary_dim, (int32_t)ffn, (float)eps};
+    ps->dims = d;
+    const int64_t H = hidden, F = ffn, L = (int64_t)layers.size();
+    TORCH_CHECK(L > 0 && (int64_t)k_caches.size() == L && (int64_t)v_caches.size() == L, "need one K and V cache per layer");
+    TORCH_CHECK(embed.dim() == 2 && embed.size(1) == H, "embed must be [vocab, H]");
+    const int64_t V = embed.size(0);
+    check_half(embed, "embed", V * H, embed);
+    check_half(lm_head, "lm_head", V * H, embed);
+    check_half(final_ln_w, "final_ln_weight", H, embed);
+    check_half(final_ln_b, "final_ln_bias", H, embed);
+    std::vector<cfpp_neox_weights> lw(L);
+    std::vector<void*> kc(L), vc(L);
+    int64_t rows = -1;
+    for (int64_t l = 0; l < L; ++l) {
+        TORCH_CHECK(layers[l].size() == 12, "each layer is 12 tensors: ln_w ln_b w_qkv b_qkv w_o b_o post_ln_w post_ln_b w_up b_up w_down b_down");
+        const int64_t numel[12] = {H, H, 3 * H * H, 3 * H, H * H, H, H, H, F * H, F, H * F, H};
+        for (int i = 0; i < 12; ++i) { check_half(layers[l][i], "layer tensor", numel[i], embed); ps->keep.push_back(layers[l][i]); }
+        const void* q[12];
+        for (int i = 0; i < 12; ++i) q[i] = layers[l][i].data_ptr();
+        lw[l] = cfpp_neox_weights{q[0], q[1], q[2], q[3], q[4], q[5], q[6], q[7], q[8], q[9], q[10], q[11]};
+        const int64_t rk = check_cache(k_caches[l], "k_cache", H, embed), rv = check_cache(v_caches[l], "v_cache", H, embed);
+        TORCH_CHECK(rk == rv && (rows < 0 || rows == rk), "all caches must have the same number of rows");
+        rows = rk;
+        kc[l] = k_caches[l].data_ptr(); vc[l] = v_caches[l].data_ptr();
+        ps->keep.push_back(k_caches[l]); ps->keep.push_back(v_caches[l]);
+    }
+    check_rope(rope_cos, "rope_cos", rows * rotary_dim, embed);
+    check_rope(rope_sin, "rope_sin", rows * rotary_dim, embed);
+    TORCH_CHECK(rope_cos.dim() == 2 && rope_cos.size(1) == rotary_dim && rope_sin.sizes() == rope_cos.sizes(),
+                "rope tables must be [positions, rotary_dim]");
+    for (const Tensor& t : {embed, final_ln_w, final_ln_b, lm_head, rope_cos, rope_sin}) ps->keep.push_back(t);
+    cfpp_neox_stack_desc desc{};
+    desc.dims = d; desc.n_layers = (int32_t)L; desc.vocab = (int32_t)V;
+    desc.layers = lw.data(); desc.embed = embed.data_ptr(); desc.final_ln_w = final_ln_w.data_ptr();
+    desc.final_ln_b = final_ln_b.data_ptr(); desc.lm_head = lm_head.data_ptr();
+    desc.k_caches = kc.data(); desc.v_caches = vc.data(); desc.cache_rows = (int32_t)rows;
+    desc.rope_cos = rope_cos.data_ptr<float>(); desc.rope_sin = rope_sin.data_ptr<float>();
+    desc.mode = (int32_t)mode;
+    c10::hip::HIPGuard guard(embed.device());
+    check_rc(cfpp_stack_create(&desc, &ps->s), "stack_create");
+    ps->vocab = V;
+    ps->device = embed.device();
+    return ps;
+}
+
+hipStream_t cur_stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+}  // namespace
+
+#define LAYER_ARGS                                                                                                     \
+    Tensor input, Tensor weight_qkv, Tensor bias_qkv, Tensor weight_o, Tensor bias_o, Tensor k_cache, Tensor v_cache, \
+        Tensor layernorm_weight, Tensor layernorm_bias, Tensor cos, Tensor sin, Tensor post_ln_weight,                \
+        Tensor post_ln_bias, Tensor mlp_up_weight, Tensor mlp_up_bias
+#define LAYER_PACK(dw, db)                                                                                              \
+    LayerArgs { input, weight_qkv, bias_qkv, weight_o, bias_o, k_cache, v_cache, layernorm_weight, layernorm_bias, cos, \
+                sin, post_ln_weight, post_ln_bias, mlp_up_weight, mlp_up_bias, dw, db }
+
+#define DEFINE_MODEL_OPS(m, MODEL)                                                                                     \
+    m.def(#MODEL "_decoder_layer", [](LAYER_ARGS, Tensor mlp_down_weight, Tensor mlp_down_bias, int64_t current_seq_len) { \
+        return decoder_layer(k##MODEL, CFPP_MODE_FUSED, LAYER_PACK(mlp_down_weight, mlp_down_bias), current_seq_len);  \
+    });                                                                                                                \
+    m.def(#MODEL "_decoder_layer_split", [](LAYER_ARGS, Tensor mlp_down_weight, Tensor mlp_down_bias, int64_t current_seq_len) { \
+        return decoder_layer(k##MODEL, CFPP_MODE_SPLIT, LAYER_PACK(mlp_down_weight, mlp_down_bias), current_seq_len);  \
+    });                                                                                                                \
+    m.def(#MODEL "_attention_only", [](LAYER_ARGS, int64_t current_seq_len) {                                          \
+        return attention_only(k##MODEL, LAYER_PACK(Tensor(), Tensor()), current_seq_len);                              \
+    });                                                                                                                \
+    m.def(#MODEL "_mlp_only", [](Tensor input, Tensor attn_output, Tensor mlp_intermediate, Tensor mlp_down_weight,    \
+                                 Tensor mlp_down_bias) {                                                               \
+        return mlp_only(k##MODEL, input, attn_output, mlp_intermediate, mlp_down_weight, mlp_down_bias);               \
+    });                                                                                                                \
+    m.def(#MODEL "_create_graph_context", [](int64_t context_id, Tensor k_cache, Tensor v_cache, Tensor weight_qkv,    \
+                                             Tensor weight_o, Tensor mlp_up_weight, Tensor mlp_down_weight,            \
+                                             int64_t max_seq_len) {                                                    \
+        create_graph_context(k##MODEL, context_id, k_cache, v_cache, weight_qkv, weight_o, mlp_up_weight,              \
+                             mlp_down_weight, max_seq_len);                                                            \
+    });                                                                                                                \
+    m.def(#MODEL "_graph_decode_step", [](int64_t context_id, Tensor input, Tensor layernorm_weight,                   \
+                                          Tensor layernorm_bias, Tensor qkv_bias, Tensor o_bias, Tensor cos, Tensor sin, \
+                                          Tensor k_cache, Tensor v_cache, Tensor post_ln_weight, Tensor post_ln_bias,  \
+                                          Tensor mlp_up_bias, Tensor mlp_down_bias, py::object current_seq_len) {      \
+        return graph_decode_step(k##MODEL, context_id, input, layernorm_weight, layernorm_bias, qkv_bias, o_bias, cos, \
+                                 sin, k_cache, v_cache, post_ln_weight, post_ln_bias, mlp_up_bias, mlp_down_bias,      \
+                                 current_seq_len);                                                                     \
+    });                                                                                                                \
+    m.def(#MODEL "_destroy_graph_context", [](int64_t context_id) { destroy_graph_context(k##MODEL, context_id); });
+
+namespace {
+const Model& kpythia_2b8 = kPythia2b8;
+const Model& kpythia_6b9 = kPythia6b9;
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    m.doc() = "MI355X (gfx950) fused GPT-NeoX / Pythia decode step";
+    DEFINE_MODEL_OPS(m, pythia_2b8)
+    DEFINE_MODEL_OPS(m, pythia_6b9)
+
+    m.def("cfpp_version", []() { return std::string(cfpp_version()); });
+    m.def("workspace_bytes", [](int64_t hidden, int64_t heads, int64_t head_dim, int64_t rotary_dim, int64_t ffn) {
+        cfpp_neox_dims d{(int32_t)hidden, (int32_t)heads, (int32_t)head_dim, (int32_t)rotary_dim, (int32_t)ffn, 1e-5f};
+        return (int64_t)cfpp_neox_workspace_bytes(&d);
+    });
+    m.def("check_workspace", [](Tensor like, int64_t hidden, int64_t heads, int64_t head_dim, int64_t rotary_dim, int64_t ffn) {
+        // reads (and clears) the device-side failure flag of the calling stream's scratch buffer
+        cfpp_neox_dims d{(int32_t)hidden, (int32_t)heads, (int32_t)head_dim, (int32_t)rotary_dim, (int32_t)ffn, 1e-5f};
+        c10::hip::HIPGuard guard(like.device());
+        hipStream_t st = cur_stream();
+        Tensor ws = workspace_for(d, like.device(), st);
+        return cfpp_workspace_check(&d, ws_ptr(ws), st);
+    });
+    m.def("lm_head", [](Tensor x, Tensor ln_w, Tensor ln_b, Tensor w, double eps) {
+        TORCH_CHECK(w.dim() == 2, "lm head weight must be [vocab, H]");
+        const int64_t V = w.size(0), H = w.size(1);
+        check_half(x, "x", H, x);
+        check_half(ln_w, "ln_weight", H, x);
+        check_half(ln_b, "ln_bias", H, x);
+        check_half(w, "weight", V * H, x);
+        c10::hip::HIPGuard guard(x.device());
+        Tensor logits = torch::empty({V}, x.options().dtype(torch::kFloat32));
+        check_rc(cfpp_neox_lm_head((int32_t)H, (int32_t)V, (float)eps, x.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(),
+                                   w.data_ptr(), logits.data_ptr<float>(), cur_stream()), "lm_head");
+        return logits;
+    });
+
+    py::class_<PyStack, std::shared_ptr<PyStack>>(m, "NeoxStack")
+        .def(py::init(&stack_create), py::arg("hidden"), py::arg("heads"), py::arg("head_dim"), py::arg("rotary_dim"),
+             py::arg("ffn"), py::arg("eps"), py::arg("layers"), py::arg("embed"), py::arg("final_ln_weight"),
+             py::arg("final_ln_bias"), py::arg("lm_head"), py::arg("k_caches"), py::arg("v_caches"), py::arg("rope_cos"),
+             py::arg("rope_sin"), py::arg("mode") = 0)
+        .def("set_state", [](PyStack& s, int64_t token, int64_t seq_len) {
+            c10::hip::HIPGuard guard(s.device);
+            check_rc(cfpp_stack_set_state(s.s, (int32_t)token, (int32_t)seq_len, cur_stream()), "set_state");
+        })
+        .def("step", [](PyStack& s) {
+            c10::hip::HIPGuard guard(s.device);
+            check_rc(cfpp_stack_step(s.s, cur_stream()), "step");
+        })
+        .def("graph_steps", [](PyStack& s, int64_t n) {
+            c10::hip::HIPGuard guard(s.device);
+            check_rc(cfpp_stack_graph_steps(s.s, (int32_t)n, cur_stream()), "graph_steps");
+        })
+        .def("logits", [](PyStack& s) {
+            float* p = nullptr;
+            check_rc(cfpp_stack_buffers(s.s, &p, nullptr, nullptr, nullptr, nullptr), "buffers");
+            return torch::from_blob(p, {s.vocab}, torch::TensorOptions().dtype(torch::kFloat32).device(s.device));
+        })
+        .def("hidden", [](PyStack& s) {
+            void* p = nullptr;
+            check_rc(cfpp_stack_buffers(s.s, nullptr, &p, nullptr, nullptr, nullptr), "buffers");
+            return torch::from_blob(p, {1, (int64_t)s.dims.hidden}, torch::TensorOptions().dtype(torch::kFloat16).device(s.device));
+        })
+        .def("state", [](PyStack& s) {
+            int32_t* p = nullptr;
+            check_rc(cfpp_stack_buffers(s.s, nullptr, nullptr, &p, nullptr, nullptr), "buffers");
+            return torch::from_blob(p, {3}, torch::TensorOptions().dtype(torch::kInt32).device(s.device));
+        })
+        .def("history", [](PyStack& s) {
+            int32_t* p = nullptr;
+            int32_t cap = 0;
+            check_rc(cfpp_stack_buffers(s.s, nullptr, nullptr, nullptr, &p, &cap), "buffers");
+            return torch::from_blob(p, {(int64_t)cap}, torch::TensorOptions().dtype(torch::kInt32).device(s.device));
+        });
+}

@@ -1,0 +1,89 @@
+"""Host-side model runner: the counterpart of the reference's full-model decode loop
+(reference tests/benchmark_decode.py:60-119 `prepare_setup`, :147-189 the per-token loop), with the
+loop body moved into one hipGraph replay per token (embedding row -> layers -> final LayerNorm ->
+LM head -> argmax all on the device)."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Sequence
+
+import torch
+
+
+@dataclass(frozen=True)
+class NeoxConfig:
+    hidden: int
+    heads: int
+    head_dim: int
+    rotary_dim: int
+    ffn: int
+    n_layers: int
+    vocab: int
+    eps: float = 1e-5
+    rope_base: float = 10000.0
+
+
+PYTHIA_2B8 = NeoxConfig(hidden=2560, heads=32, head_dim=80, rotary_dim=20, ffn=10240, n_layers=32, vocab=50304)
+PYTHIA_6B9 = NeoxConfig(hidden=4096, heads=32, head_dim=128, rotary_dim=32, ffn=16384, n_layers=32, vocab=50432)
+
+# order of the 12 per-layer tensors (same set the reference pulls out of the HF module,
+# tests/benchmark_decode.py:83-96)
+layer_tensor_order = ("ln_w", "ln_b", "w_qkv", "b_qkv", "w_o", "b_o",
+                      "post_ln_w", "post_ln_b", "w_up", "b_up", "w_down", "b_down")
+
+
+def rope_tables(positions: int, rotary_dim: int, base: float = 10000.0, device="cuda"):
+    """fp32 cos/sin tables `[positions, rotary_dim]`, emb = cat(freqs, freqs)
+    (reference tests/benchmark_decode.py:39-57)."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, rotary_dim, 2, dtype=torch.float64) / rotary_dim))
+    freqs = torch.arange(positions, dtype=torch.float64)[:, None] * inv_freq[None, :]
+    emb = torch.cat([freqs, freqs], dim=-1)
+    return emb.cos().float().to(device).contiguous(), emb.sin().float().to(device).contiguous()
+
+
+class NeoxDecoder:
+    """Greedy batch-1 decoder over device-resident weights and KV caches.
+
+    `layers` is a list of dicts keyed by `layer_tensor_order`; caches are `[cache_rows, H]` fp16
+    (HF `past_key_values` `[1, heads, S, D]` maps to this layout by `permute(0,2,1,3).reshape(S, H)`,
+    reference tests/benchmark_decode.py:99-108)."""
+
+    def __init__(self, cfg: NeoxConfig, layers: Sequence[Dict[str, torch.Tensor]], embed: torch.Tensor,
+                 final_ln_w: torch.Tensor, final_ln_b: torch.Tensor, lm_head: torch.Tensor,
+                 k_caches: List[torch.Tensor], v_caches: List[torch.Tensor], mode: str = "fused"):
+        from . import _clusterfusion as native
+        self.cfg = cfg
+        rows = k_caches[0].shape[0]
+        self.cos, self.sin = rope_tables(rows, cfg.rotary_dim, cfg.rope_base, device=embed.device)
+        packed = [[w[k].reshape(-1) if w[k].dim() == 1 else w[k] for k in layer_tensor_order] for w in layers]
+        self._stack = native.NeoxStack(cfg.hidden, cfg.heads, cfg.head_dim, cfg.rotary_dim, cfg.ffn, cfg.eps,
+                                       packed, embed, final_ln_w, final_ln_b, lm_head, list(k_caches), list(v_caches),
+                                       self.cos, self.sin, {"fused": 0, "split": 1}[mode])
+
+    def set_state(self, token: int, seq_len: int):
+        self._stack.set_state(int(token), int(seq_len))
+
+    def step(self):
+        """One eager decode step (one launch per kernel)."""
+        self._stack.step()
+
+    def graph_steps(self, n: int):
+        """`n` decode steps, each one replay of the captured hipGraph."""
+        self._stack.graph_steps(int(n))
+
+    @property
+    def logits(self) -> torch.Tensor:
+        return self._stack.logits()
+
+    @property
+    def hidden(self) -> torch.Tensor:
+        return self._stack.hidden()
+
+    @property
+    def state(self) -> torch.Tensor:
+        """int32 `[token, seq_len, steps_done]` on the device."""
+        return self._stack.state()
+
+    def generated(self) -> List[int]:
+        n = int(self.state[2].item())
+        return self._stack.history()[:n].tolist()

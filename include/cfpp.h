@@ -1,0 +1,193 @@
+/*
+ * cfpp.h - C ABI of the MI355X (gfx950) GPT-NeoX / Pythia fused decode-step library.
+ *
+ * Plain C: raw device pointers, sizes and a hipStream_t passed as void*.  No torch types.
+ * The PyTorch extension (`clusterfusion._clusterfusion`) and any other host (a C++ serving
+ * loop, ctypes) bind exactly these entry points.
+ *
+ * Conventions for every call that returns `int`:
+ *   0  success; <0 a `cfpp_status` argument error (nothing was launched); >0 a hipError_t.
+ * No entry point throws or synchronises the device; only the ones whose comment says so
+ * allocate device memory (context / stack creation).  All launches go to the given stream.
+ *
+ * Tensor contract (same as the reference's dispatch code,
+ * include/5090/pythia_2b8/pythia_kernel_dispatch.cu:4-75): fp16 row-major contiguous;
+ * weights in nn.Linear layout [out, in]; W_qkv / b_qkv head-interleaved [head][q|k|v][D]
+ * (reference include/5090/pythia_2b8/config.h:14-18); K/V caches [rows, H] with head-major
+ * columns; cos/sin fp32 with at least rotary_dim entries per position.
+ */
+#ifndef CFPP_H
+#define CFPP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum cfpp_status {
+    CFPP_OK = 0,
+    CFPP_ERR_NULL = -1,        /* a required pointer is NULL */
+    CFPP_ERR_DIMS = -2,        /* unsupported dimensions */
+    CFPP_ERR_SEQ = -3,         /* seq_len < 0 or seq_len > cache rows available */
+    CFPP_ERR_WORKSPACE = -4,   /* workspace too small or misaligned */
+    CFPP_ERR_CONTEXT = -5,     /* unknown / duplicate context id */
+    CFPP_ERR_MODE = -6,        /* unknown mode */
+    CFPP_ERR_DEVICE = -7,      /* device-side failure flag raised (bounded wait expired, bad seq_len) */
+    CFPP_ERR_ALIGN = -8        /* a tensor pointer is not 16-byte aligned */
+} cfpp_status;
+
+/* Layer geometry.  Pythia-2.8B = {2560,32,80,20,10240,1e-5}, Pythia-6.9B = {4096,32,128,32,16384,1e-5}
+ * (reference include/5090/pythia_2b8/config.h:6-12, include/5090/pythia_6b9/config.h:6-12).
+ * Supported: hidden == heads*head_dim, hidden % 8 == 0, hidden <= 8192, head_dim % 8 == 0,
+ * head_dim <= 128, rotary_dim even and <= head_dim, ffn % 8 == 0. */
+typedef struct cfpp_neox_dims {
+    int32_t hidden, heads, head_dim, rotary_dim, ffn;
+    float eps;
+} cfpp_neox_dims;
+
+/* The 12 per-layer tensors (reference tests/benchmark_decode.py:83-96 extracts the same set). */
+typedef struct cfpp_neox_weights {
+    const void *ln_w, *ln_b;            /* input LayerNorm [H] */
+    const void *w_qkv, *b_qkv;          /* [3H,H], [3H] head-interleaved */
+    const void *w_o, *b_o;              /* [H,H], [H] */
+    const void *post_ln_w, *post_ln_b;  /* post-attention LayerNorm [H] (feeds the MLP; parallel residual) */
+    const void *w_up, *b_up;            /* [F,H], [F] */
+    const void *w_down, *b_down;        /* [H,F], [H] */
+} cfpp_neox_weights;
+
+/* Per-call tensors.  `seq_len` counts valid cache rows BEFORE the append (reference
+ * pythia_kernel_dispatch.cu:68-75).  If `d_seq_len` is non-NULL the kernels read the length
+ * from that device int32 instead (needed for hipGraph replay) and cos/sin are indexed by it:
+ * row = cos + seq_len * rope_stride (rope_stride 0 = the given row is the current position). */
+typedef struct cfpp_neox_io {
+    const void* input;       /* [H] fp16, read only */
+    void* output;            /* [H] fp16 */
+    void* k_new;             /* [heads*D] fp16: rotated K of the new token */
+    void* v_new;             /* [heads*D] fp16 */
+    void* k_cache;           /* [cache_rows, H] fp16; row seq_len is written if cache_rows > seq_len */
+    void* v_cache;
+    int32_t cache_rows;
+    const float* cos;
+    const float* sin;
+    int32_t rope_stride;
+    int32_t seq_len;
+    const int32_t* d_seq_len;
+    int32_t max_seq_len;     /* upper bound used to size the KV split when d_seq_len is given; 0 = cache_rows */
+    void* attn_output;       /* split API only: [H] fp16 = W_o attn + b_o */
+    void* mlp_intermediate;  /* split API only: [F] fp16 = gelu(W_up ln2(x) + b_up) */
+} cfpp_neox_io;
+
+typedef enum cfpp_mode {
+    CFPP_MODE_FUSED = 0,     /* one persistent launch with device-wide barriers between the stages */
+    CFPP_MODE_SPLIT = 1      /* one plain launch per stage; the kernel boundary is the barrier */
+} cfpp_mode;
+
+const char* cfpp_status_str(int status);
+const char* cfpp_version(void);
+
+/* Bytes of device scratch one layer call needs (256-byte aligned; zero it once before first use). */
+size_t cfpp_neox_workspace_bytes(const cfpp_neox_dims* dims);
+
+/* Full decoder-layer decode step.
+ * Replaces pythia_2b8_decoder_layer_sm120 / pythia_6b9_decoder_layer_sm120 (reference
+ * include/pybind.cpp:109-129,183-203; include/5090/pythia_2b8/pythia_kernel_dispatch.cu:4-251) in
+ * CFPP_MODE_FUSED and pythia_2b8_decoder_layer_split_sm120 (include/pybind.cpp:132-151;
+ * pythia_kernel_dispatch_split.cu:18-218) in CFPP_MODE_SPLIT. */
+int cfpp_neox_layer_decode(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io,
+                           int mode, void* workspace, size_t workspace_bytes, void* stream);
+
+/* First half of the split API: LN, QKV, RoPE, append, attention, O-proj (+b_o) -> io->attn_output,
+ * and MLP-up + GELU -> io->mlp_intermediate; k_new / v_new / cache row as in the full layer.
+ * `w->w_down`, `w->b_down` and `io->output` are ignored.
+ * Replaces pythia_2b8_attention_only_sm120 (reference include/pybind.cpp:154-171;
+ * pythia_kernel_dispatch_split.cu:225-359). */
+int cfpp_neox_attention_mlp_up(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
+/* Second half: output = input + attn_output + W_down mlp_intermediate + b_down.
+ * Replaces pythia_2b8_mlp_only_sm120 (reference include/pybind.cpp:174-180;
+ * pythia_kernel_dispatch_split.cu:364-426). */
+int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void* attn_output,
+                       const void* mlp_intermediate, const void* w_down, const void* b_down, void* output,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- per-layer decode contexts (persistent buffers keyed by an integer id) --------------------
+ * Replaces PythiaGraphContext + create / graph_decode_step / destroy (reference
+ * include/5090/pythia_2b8/pythia_kernel_dispatch_graph.cu:50-294 and the 6.9B twin;
+ * include/pybind.cpp:206-267).  `family` separates the id spaces the reference keeps in two maps
+ * (g_contexts / g_contexts_6b9): 0 = 2.8B ops, 1 = 6.9B ops, any other int = caller-defined. */
+typedef struct cfpp_ctx_buffers {
+    void* output;   /* [H] fp16, context-owned, overwritten by the next step */
+    void* k_new;    /* [heads*D] fp16 */
+    void* v_new;    /* [heads*D] fp16 */
+} cfpp_ctx_buffers;
+
+/* Allocates the context's output buffers and workspace on the current device (hipMalloc).
+ * Duplicate id: the old context is destroyed and replaced (the reference silently overwrites). */
+int cfpp_ctx_create(int family, int64_t id, const cfpp_neox_dims* dims, const void* w_qkv, const void* w_o,
+                    const void* w_up, const void* w_down, void* k_cache, void* v_cache, int32_t cache_rows,
+                    int32_t max_seq_len, cfpp_ctx_buffers* out_buffers);
+
+/* One decode step on the context's buffers; `w` carries the small vectors (the four matrices in it
+ * must be NULL or equal to those given at create), `io->output/k_new/v_new` are ignored, and
+ * io->k_cache / v_cache must equal the create-time pointers (CFPP_ERR_CONTEXT otherwise).
+ * Unknown id -> CFPP_ERR_CONTEXT.  Allocates nothing, never synchronises: capturable in a hipGraph
+ * when io->d_seq_len is used. */
+int cfpp_ctx_step(int family, int64_t id, const cfpp_neox_weights* w, const cfpp_neox_io* io, int mode,
+                  void* stream, cfpp_ctx_buffers* out_buffers);
+
+/* Frees the context's buffers; unknown id is a no-op returning CFPP_OK. */
+int cfpp_ctx_destroy(int family, int64_t id);
+
+/* Reads and clears the device-side failure flag of a workspace (synchronises `stream`).
+ * Returns CFPP_OK or CFPP_ERR_DEVICE.  For tests and debugging; not on the hot path. */
+int cfpp_workspace_check(const cfpp_neox_dims* dims, void* workspace, void* stream);
+
+/* ---- whole-model greedy decode (our counterpart of the reference's Python decode loop,
+ * tests/benchmark_decode.py:147-189: embedding row -> layers -> final LayerNorm -> LM head ->
+ * argmax), captured once into a hipGraph and replayed per token ------------------------------- */
+typedef struct cfpp_neox_stack_desc {
+    cfpp_neox_dims dims;
+    int32_t n_layers;
+    int32_t vocab;
+    const cfpp_neox_weights* layers;   /* host array [n_layers] of device pointers */
+    const void* embed;                 /* [vocab, H] fp16 */
+    const void* final_ln_w;            /* [H] fp16 */
+    const void* final_ln_b;
+    const void* lm_head;               /* [vocab, H] fp16 */
+    void* const* k_caches;             /* host array [n_layers] of device pointers [cache_rows, H] */
+    void* const* v_caches;
+    int32_t cache_rows;
+    const float* rope_cos;             /* [cache_rows, rotary_dim] fp32 table indexed by position */
+    const float* rope_sin;
+    int32_t mode;                      /* cfpp_mode used for every layer */
+} cfpp_neox_stack_desc;
+
+typedef struct cfpp_neox_stack cfpp_neox_stack;   /* opaque */
+
+/* Allocates state (device int32 seq_len + token, hidden ping-pong, logits, workspace). */
+int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out);
+/* Sets the device-resident (token, seq_len) the next step starts from (async on `stream`). */
+int cfpp_stack_set_state(cfpp_neox_stack* s, int32_t token, int32_t seq_len, void* stream);
+/* One decode step launched eagerly: consumes (token, seq_len), appends K/V rows, writes logits,
+ * then stores argmax as the new token and seq_len+1. */
+int cfpp_stack_step(cfpp_neox_stack* s, void* stream);
+/* Captures one step into a hipGraph (first call) and replays it `n_steps` times on `stream`. */
+int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream);
+/* Device pointers for inspection: logits fp32 [vocab], hidden fp16 [H] after the last layer,
+ * state int32[3] = {token, seq_len, steps done}, token history int32 [history_capacity]. */
+int cfpp_stack_buffers(cfpp_neox_stack* s, float** logits, void** hidden, int32_t** state,
+                       int32_t** history, int32_t* history_capacity);
+int cfpp_stack_destroy(cfpp_neox_stack* s);
+
+/* Final LayerNorm + LM-head GEMV: logits[v] = W[v,:] . LN(x) (no bias), fp32 logits.
+ * Counterpart of F.layer_norm + embed_out in the reference loop (tests/benchmark_decode.py:180-187). */
+int cfpp_neox_lm_head(int32_t hidden, int32_t vocab, float eps, const void* x, const void* ln_w,
+                      const void* ln_b, const void* w, float* logits, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CFPP_H */
