@@ -73,6 +73,35 @@ __device__ __forceinline__ u32x4 ld_stream16(const void* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }
 __device__ __forceinline__ u32x4 ld16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+
+// Device-coherent accessors for values that cross workgroups inside one launch.  Every XCD has its
+// own L2, so plain stores may sit dirty in one L2 while another XCD reads a stale line.  Relaxed
+// agent-scope atomics compile to sc1 stores (write through) and sc1 loads (miss in the caches), which
+// makes the hand-off coherent without agent-scope fences; those fences write back / invalidate the
+// whole L2 and cost far more than the data they protect.  The producer drains its stores
+// (s_waitcnt 0) before it bumps the counter the consumer polls.
+__device__ __forceinline__ void st_agent(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(half_t* p, half_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(uint32_t* p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_agent(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ u32x4 ld_agent16(const void* p) {
+    const uint64_t* q = reinterpret_cast<const uint64_t*>(p);
+    const uint64_t a = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint64_t b = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    u32x4 r = {(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
+    return r;
+}
+// all memory operations this wave has issued are complete
+__device__ __forceinline__ void drain_memory_ops() { __builtin_amdgcn_s_waitcnt(0); }
+
 __device__ __forceinline__ half2_t as_h2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
 __device__ __forceinline__ uint32_t as_u32(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
 
@@ -134,14 +163,16 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // ------------------------------------------------------------------------------------------------
 // device-wide synchronisation (bounded spins; a timeout raises a status flag and falls through)
 // ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ void counter_add_release(int* ctr, int v) {
-    __hip_atomic_fetch_add(ctr, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+// arrive: the caller has drained its stores (and, for a workgroup-wide arrival, synchronised the workgroup)
+__device__ __forceinline__ void counter_add(int* ctr, int v) {
+    __hip_atomic_fetch_add(ctr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// one thread spins; the whole workgroup leaves together and sees the other workgroups' writes
+// one thread polls; the whole workgroup leaves together.  Data published before the arrivals must be
+// read with ld_agent / ld_agent16.
 __device__ __forceinline__ void grid_wait(int* ctr, int target, int* status) {
     if (threadIdx.x == 0) {
         long long spins = 0;
-        while (__hip_atomic_load(ctr, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
             __builtin_amdgcn_s_sleep(1);
             if (++spins > kSpinLimit) {
                 __hip_atomic_fetch_or(status, kStatusSpin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -150,7 +181,7 @@ __device__ __forceinline__ void grid_wait(int* ctr, int target, int* status) {
         }
     }
     __syncthreads();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
 __device__ __forceinline__ int load_seq_len(const LayerParams& p) {
@@ -279,7 +310,7 @@ __device__ __forceinline__ void stage_a_qkv(const LayerParams& p, const half2_t 
     float* __restrict__ dst = p.qkv_raw;
     gemv_rows_auto<NCH>(p.w_qkv, p.H, gw, nw, 3 * p.H, x1, lane,
                         [&](int r) { return (float)bias[r]; },
-                        [&](int r, float v, float b) { if (lane == 0) dst[r] = v + b; });
+                        [&](int r, float v, float b) { if (lane == 0) st_agent(dst + r, v + b); });
 }
 template <int NCH>
 __device__ __forceinline__ void stage_a_up(const LayerParams& p, const half2_t (&x2)[NCH][4], int gw, int nw, int lane) {
@@ -287,7 +318,7 @@ __device__ __forceinline__ void stage_a_up(const LayerParams& p, const half2_t (
     half_t* __restrict__ dst = p.inter;
     gemv_rows_auto<NCH>(p.w_up, p.H, gw, nw, p.F, x2, lane,
                         [&](int r) { return (float)bias[r]; },
-                        [&](int r, float v, float b) { if (lane == 0) dst[r] = (half_t)gelu_tanh(v + b); });
+                        [&](int r, float v, float b) { if (lane == 0) st_agent(dst + r, (half_t)gelu_tanh(v + b)); });
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -298,10 +329,10 @@ __device__ __forceinline__ void stage_a_up(const LayerParams& p, const half2_t (
 // rot/2 <= d < rot -> v[d] cos[d] + v[d-rot/2] sin[d]; d >= rot passes through.
 __device__ __forceinline__ float rope_elem(const float* __restrict__ v, int d, int rot,
                                            const float* __restrict__ cs, const float* __restrict__ sn) {
-    const float a = v[d];
+    const float a = ld_agent(v + d);
     if (d >= rot) return a;
     const int hr = rot >> 1;
-    return d < hr ? a * cs[d] - v[d + hr] * sn[d] : a * cs[d] + v[d - hr] * sn[d];
+    return d < hr ? a * cs[d] - ld_agent(v + d + hr) * sn[d] : a * cs[d] + ld_agent(v + d - hr) * sn[d];
 }
 
 struct AttnShared {
@@ -334,7 +365,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             kf[j] = act ? rope_elem(raw + D, d0 + j, p.rot, cs, sn) : 0.f;
-            vf[j] = act ? raw[2 * D + d0 + j] : 0.f;
+            vf[j] = act ? ld_agent(raw + 2 * D + d0 + j) : 0.f;
         }
         const u32x4 kp = pack8(kf), vp = pack8(vf);
         unpack8(kp, kf); unpack8(vp, vf);      // attend over the fp16 values the cache will hold
@@ -440,29 +471,32 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
             L += sh.l[w] * sc;
             A += sh.acc[w][threadIdx.x] * sc;
         }
-        p.part_acc[item * D + threadIdx.x] = A;
-        if (threadIdx.x == 0) { p.part_ml[item * 2] = M; p.part_ml[item * 2 + 1] = L; }
+        st_agent(p.part_acc + item * D + threadIdx.x, A);
+        if (threadIdx.x == 0) { st_agent(p.part_ml + item * 2, M); st_agent(p.part_ml + item * 2 + 1, L); }
     }
-    __threadfence();
+    drain_memory_ops();
     __syncthreads();
     if (threadIdx.x == 0) {
-        const int old = __hip_atomic_fetch_add(p.head_cnt + head, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const int old = __hip_atomic_fetch_add(p.head_cnt + head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         sh.last = (old == p.nsplit - 1);
     }
     __syncthreads();
     if (sh.last) {
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        if ((int)threadIdx.x < D) {
+        // the last workgroup of this head merges the splits in split order; two dims per thread
+        const int t2 = threadIdx.x * 2;
+        if (t2 < D) {
             const size_t hb = (size_t)head * p.nsplit;
             float M = kNegBig;
-            for (int i = 0; i < p.nsplit; ++i) M = fmaxf(M, p.part_ml[(hb + i) * 2]);
-            float L = 0.f, A = 0.f;
+            for (int i = 0; i < p.nsplit; ++i) M = fmaxf(M, ld_agent(p.part_ml + (hb + i) * 2));
+            float L = 0.f, A0 = 0.f, A1 = 0.f;
             for (int i = 0; i < p.nsplit; ++i) {
-                const float sc = fast_exp2(p.part_ml[(hb + i) * 2] - M);
-                L += p.part_ml[(hb + i) * 2 + 1] * sc;
-                A += p.part_acc[(hb + i) * D + threadIdx.x] * sc;
+                const float sc = fast_exp2(ld_agent(p.part_ml + (hb + i) * 2) - M);
+                L += ld_agent(p.part_ml + (hb + i) * 2 + 1) * sc;
+                A0 += ld_agent(p.part_acc + (hb + i) * D + t2) * sc;
+                A1 += ld_agent(p.part_acc + (hb + i) * D + t2 + 1) * sc;
             }
-            p.attn_vec[(size_t)head * D + threadIdx.x] = (half_t)(A / L);
+            const half2_t o = {(half_t)(A0 / L), (half_t)(A1 / L)};
+            st_agent(reinterpret_cast<uint32_t*>(p.attn_vec + (size_t)head * D + t2), as_u32(o));
         }
         if (threadIdx.x == 0) __hip_atomic_store(p.head_cnt + head, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -518,7 +552,7 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, i
             if (col < c.K2) { wp[i] = c.W2 + col; wstride[i] = c.K2; xp = c.x2 + col; }
         }
         u32x4 xv = {0u, 0u, 0u, 0u};
-        if (xp) xv = ld16(xp);
+        if (xp) xv = ld_agent16(xp);
         xs[i][0] = as_h2(xv.x); xs[i][1] = as_h2(xv.y); xs[i][2] = as_h2(xv.z); xs[i][3] = as_h2(xv.w);
     }
 

@@ -32,7 +32,8 @@ __global__ __launch_bounds__(NWV * 64) void k_stage_a(LayerParams p, int do_qkv,
     if (do_up) stage_a_up<NCH>(p, x2, gw, nw, lane);
 }
 
-__global__ __launch_bounds__(256) void k_stage_b(LayerParams p) {
+// launched with the same workgroup size as the fused kernel so that both modes add in the same order
+__global__ __launch_bounds__(kMaxWaves * 64) void k_stage_b(LayerParams p) {
     __shared__ AttnShared sh;
     const int S = load_seq_len(p);
     const int nitems = p.heads * p.nsplit;
@@ -67,22 +68,24 @@ __global__ __launch_bounds__(NWV * 64) void k_fused(LayerParams p, int KS, int R
         half2_t x1[NCH][4], x2[NCH][4];
         load_ln_pair<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, lane, x1, x2);
         stage_a_qkv<NCH>(p, x1, gw, nw, lane);
-        if (lane == 0) counter_add_release(epoch, 1);
+        drain_memory_ops();
+        if (lane == 0) counter_add(epoch, 1);
         stage_a_up<NCH>(p, x2, gw, nw, lane);
     }
     grid_wait(epoch, nw, status);
     const int nitems = p.heads * p.nsplit;
     for (int item = blockIdx.x; item < nitems; item += G)
         attention_item(p, item / p.nsplit, item % p.nsplit, S, sha);
+    drain_memory_ops();
     __syncthreads();
-    if (threadIdx.x == 0) counter_add_release(epoch, NWV);
+    if (threadIdx.x == 0) counter_add(epoch, NWV);
     grid_wait(epoch, 2 * nw, status);
     {
         const StageC c = make_stage_c(p);
         stage_c_rows<CPW>(c, blockIdx.x, G, KS, RG, shc);
     }
     if (threadIdx.x == 0) {
-        const int old = __hip_atomic_fetch_add(exitc, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const int old = __hip_atomic_fetch_add(exitc, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (old == G - 1) {
             __hip_atomic_store(epoch, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(exitc, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -398,7 +401,7 @@ int run_split(const Plan& pl, LayerParams& p, bool full_layer, hipStream_t st) {
     int rc = launch_stage_a(pl, p, grid, 1, 1, st);
     if (rc) return rc;
     int bgrid = p.heads * p.nsplit;
-    hipLaunchKernelGGL(k_stage_b, dim3(bgrid), dim3(256), 0, st, p);
+    hipLaunchKernelGGL(k_stage_b, dim3(bgrid), dim3(pl.nwv * 64), 0, st, p);
     if ((rc = launch_check())) return rc;
     (void)full_layer;
     return launch_stage_c(pl, p, grid, st);

@@ -11,8 +11,8 @@
 //     as `[positions, rotary_dim]` tables), which makes the step replayable from a captured HIP graph.
 // This file contains no device code; torch is used for tensors, streams and exceptions only.
 #include <torch/extension.h>
-#include <c10/hip/HIPStream.h>
-#include <c10/hip/HIPGuard.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <map>
 #include <memory>
@@ -136,13 +136,13 @@ std::tuple<Tensor, Tensor, Tensor> decoder_layer(const Model& m, int mode, const
     cfpp_neox_io io;
     fill_weights(d, a, true, &w);
     fill_io(d, a, seq_len, &io);
-    c10::hip::HIPGuard guard(a.input.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(a.input.device());
     auto opts = a.input.options();
     Tensor out = torch::empty({1, d.hidden}, opts);
     Tensor k = torch::empty({1, d.heads, d.head_dim}, opts);
     Tensor v = torch::empty({1, d.heads, d.head_dim}, opts);
     io.output = out.data_ptr(); io.k_new = k.data_ptr(); io.v_new = v.data_ptr();
-    hipStream_t st = c10::hip::getCurrentHIPStream().stream();
+    hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     Tensor ws = workspace_for(d, a.input.device(), st);
     check_rc(cfpp_neox_layer_decode(&d, &w, &io, mode, ws_ptr(ws), cfpp_neox_workspace_bytes(&d), st), m.name);
     return std::make_tuple(out, k, v);
@@ -154,7 +154,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> attention_only(const Model& m, const 
     cfpp_neox_io io;
     fill_weights(d, a, false, &w);
     fill_io(d, a, seq_len, &io);
-    c10::hip::HIPGuard guard(a.input.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(a.input.device());
     auto opts = a.input.options();
     Tensor attn = torch::empty({1, d.hidden}, opts);
     Tensor inter = torch::empty({d.ffn}, opts);
@@ -162,7 +162,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> attention_only(const Model& m, const 
     Tensor v = torch::empty({1, d.heads, d.head_dim}, opts);
     io.attn_output = attn.data_ptr(); io.mlp_intermediate = inter.data_ptr();
     io.k_new = k.data_ptr(); io.v_new = v.data_ptr();
-    hipStream_t st = c10::hip::getCurrentHIPStream().stream();
+    hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     Tensor ws = workspace_for(d, a.input.device(), st);
     check_rc(cfpp_neox_attention_mlp_up(&d, &w, &io, ws_ptr(ws), cfpp_neox_workspace_bytes(&d), st), m.name);
     return std::make_tuple(attn, inter, k, v);
@@ -175,9 +175,9 @@ Tensor mlp_only(const Model& m, Tensor input, Tensor attn_output, Tensor inter, 
     check_half(inter, "mlp_intermediate", d.ffn, input);
     check_half(down_w, "mlp_down_weight", (int64_t)d.hidden * d.ffn, input);
     check_half(down_b, "mlp_down_bias", d.hidden, input);
-    c10::hip::HIPGuard guard(input.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
     Tensor out = torch::empty({1, d.hidden}, input.options());
-    hipStream_t st = c10::hip::getCurrentHIPStream().stream();
+    hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_rc(cfpp_neox_mlp_down(&d, input.data_ptr(), attn_output.data_ptr(), inter.data_ptr(), down_w.data_ptr(),
                                 down_b.data_ptr(), out.data_ptr(), nullptr, 0, st), m.name);
     return out;
@@ -203,7 +203,7 @@ void create_graph_context(const Model& m, int64_t id, Tensor k_cache, Tensor v_c
     check_half(w_down, "mlp_down_weight", H * F, k_cache);
     const int64_t rows = std::min(rows_k, rows_v);
     TORCH_CHECK(max_seq_len > 0 && max_seq_len <= rows, "max_seq_len ", max_seq_len, " must be in [1, cache rows = ", rows, "]");
-    c10::hip::HIPGuard guard(k_cache.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(k_cache.device());
     cfpp_ctx_buffers b{};
     check_rc(cfpp_ctx_create(m.family, id, &d, w_qkv.data_ptr(), w_o.data_ptr(), w_up.data_ptr(), w_down.data_ptr(),
                              k_cache.data_ptr(), v_cache.data_ptr(), (int32_t)rows, (int32_t)max_seq_len, &b),
@@ -269,8 +269,8 @@ std::tuple<Tensor, Tensor, Tensor> graph_decode_step(const Model& m, int64_t id,
         TORCH_CHECK(s >= 0 && s <= rows, "current_seq_len ", s, " out of range for ", rows, " cache rows");
         io.seq_len = (int32_t)s;
     }
-    c10::hip::HIPGuard guard(input.device());
-    hipStream_t st = c10::hip::getCurrentHIPStream().stream();
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+    hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_rc(cfpp_ctx_step(m.family, id, &w, &io, CFPP_MODE_FUSED, st, nullptr), "graph_decode_step");
     return std::make_tuple(c.output, c.k_new, c.v_new);
 }
@@ -336,14 +336,14 @@ std::shared_ptr<PyStack> stack_create(int64_t hidden, int64_t heads, int64_t hea
     desc.k_caches = kc.data(); desc.v_caches = vc.data(); desc.cache_rows = (int32_t)rows;
     desc.rope_cos = rope_cos.data_ptr<float>(); desc.rope_sin = rope_sin.data_ptr<float>();
     desc.mode = (int32_t)mode;
-    c10::hip::HIPGuard guard(embed.device());
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(embed.device());
     check_rc(cfpp_stack_create(&desc, &ps->s), "stack_create");
     ps->vocab = V;
     ps->device = embed.device();
     return ps;
 }
 
-hipStream_t cur_stream() { return c10::hip::getCurrentHIPStream().stream(); }
+hipStream_t cur_stream() { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
 
 }  // namespace
 
@@ -403,7 +403,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("check_workspace", [](Tensor like, int64_t hidden, int64_t heads, int64_t head_dim, int64_t rotary_dim, int64_t ffn) {
         // reads (and clears) the device-side failure flag of the calling stream's scratch buffer
         cfpp_neox_dims d{(int32_t)hidden, (int32_t)heads, (int32_t)head_dim, (int32_t)rotary_dim, (int32_t)ffn, 1e-5f};
-        c10::hip::HIPGuard guard(like.device());
+        c10::hip::HIPGuardMasqueradingAsCUDA guard(like.device());
         hipStream_t st = cur_stream();
         Tensor ws = workspace_for(d, like.device(), st);
         return cfpp_workspace_check(&d, ws_ptr(ws), st);
@@ -415,7 +415,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         check_half(ln_w, "ln_weight", H, x);
         check_half(ln_b, "ln_bias", H, x);
         check_half(w, "weight", V * H, x);
-        c10::hip::HIPGuard guard(x.device());
+        c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
         Tensor logits = torch::empty({V}, x.options().dtype(torch::kFloat32));
         check_rc(cfpp_neox_lm_head((int32_t)H, (int32_t)V, (float)eps, x.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(),
                                    w.data_ptr(), logits.data_ptr<float>(), cur_stream()), "lm_head");
@@ -428,15 +428,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
              py::arg("final_ln_bias"), py::arg("lm_head"), py::arg("k_caches"), py::arg("v_caches"), py::arg("rope_cos"),
              py::arg("rope_sin"), py::arg("mode") = 0)
         .def("set_state", [](PyStack& s, int64_t token, int64_t seq_len) {
-            c10::hip::HIPGuard guard(s.device);
+            c10::hip::HIPGuardMasqueradingAsCUDA guard(s.device);
             check_rc(cfpp_stack_set_state(s.s, (int32_t)token, (int32_t)seq_len, cur_stream()), "set_state");
         })
         .def("step", [](PyStack& s) {
-            c10::hip::HIPGuard guard(s.device);
+            c10::hip::HIPGuardMasqueradingAsCUDA guard(s.device);
             check_rc(cfpp_stack_step(s.s, cur_stream()), "step");
         })
         .def("graph_steps", [](PyStack& s, int64_t n) {
-            c10::hip::HIPGuard guard(s.device);
+            c10::hip::HIPGuardMasqueradingAsCUDA guard(s.device);
             check_rc(cfpp_stack_graph_steps(s.s, (int32_t)n, cur_stream()), "graph_steps");
         })
         .def("logits", [](PyStack& s) {
