@@ -5,14 +5,14 @@
 // scheme, include/5090/pythia_2b8/kernel.cuh:51-949):
 //
 //   stage A  LayerNorm statistics in registers of every wave; one wave streams whole weight rows of
-//            W_qkv (then W_up) with 16-byte lane loads, 512 contiguous halfs per wave-load, fp32
-//            accumulation through v_dot2_f32_f16, a DPP row reduction, and a scalar epilogue
-//            (bias -> raw q/k/v in fp32, or bias -> tanh-GELU -> fp16 intermediate).
-//   stage B  split-KV single-query attention: one workgroup per (head, KV split); 16 lanes per cache
-//            row, exp2-domain online softmax in fp32, fp32 partials in scratch, and the last
-//            workgroup to finish a head merges that head's partials in a fixed order.
-//            RoPE is applied when q / k are read from the raw fp32 scratch; the (head, split 0)
-//            workgroup appends the rotated K and V to the cache and returns them.
+//            W_qkv (then W_up) with 16-byte non-temporal lane loads, 512 contiguous halfs per
+//            wave-load, fp32 accumulation through v_dot2_f32_f16, a DPP row reduction, and a scalar
+//            epilogue (bias -> raw q/k/v in fp32, or bias -> tanh-GELU -> fp16 intermediate).
+//   stage B  split-KV single-query attention: one wave per (head, KV split); 16 lanes per cache
+//            row, exp2-domain online softmax in fp32, fp32 partials in scratch, and the last wave
+//            to finish a head merges that head's partials in split order.  RoPE is applied when
+//            q / k are read from the raw fp32 scratch; the (head, split 0) wave appends the rotated
+//            K and V to the cache and returns them.
 //   stage C  out = x + b_o + b_down + W_o attn + W_down h as one GEMV over the concatenated input;
 //            the K dimension is split over the waves of a workgroup (the activation slice lives in
 //            registers), rows are split over workgroups, and a fixed-order LDS reduction finishes
@@ -32,13 +32,23 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
 constexpr int kChunk = 512;            // halfs covered by one wave-wide 16-byte load
-constexpr int kMaxSplit = 32;          // KV splits per head
+constexpr int kMaxSplit = 64;          // KV splits per head (upper bound; the effective count follows seq_len)
+constexpr int kSplitRows = 64;         // target cache rows per (head, split) item
 constexpr int kMaxWaves = 16;          // waves per workgroup
-constexpr int kRowBatch = 16;          // stage-C rows reduced per LDS round
+constexpr int kRowBatch = 32;          // stage-C rows per workgroup pass
+constexpr int kUpRpi = 2;              // MLP-up rows per dynamically scheduled task
 constexpr float kNegBig = -1.0e30f;
-constexpr long long kSpinLimit = 1LL << 20;   // bounded device-side waits (order of a second)
+constexpr int kSpinLimit = 1 << 20;    // bounded device-side waits (order of a second)
 
 enum : int { kStatusSpin = 1, kStatusSeq = 2 };
+// counters in LayerParams::bar (self-resetting: the last workgroup to leave zeroes them)
+enum BarSlot : int {
+    kBarQkv = 0,      // streaming waves that have written their QKV rows
+    kBarUp = 1,       // streaming waves that have written their MLP-up rows
+    kBarHeads = 2,    // heads whose attention output is merged
+    kBarExit = 3,     // workgroups that have finished
+    kBarStatus = 4    // failure flags (kStatusSpin, kStatusSeq); not reset by the kernels
+};
 
 struct LayerParams {
     int H, heads, D, rot, F;
@@ -51,20 +61,28 @@ struct LayerParams {
     int rope_stride;
     int seq_len;
     const int* d_seq_len;
-    int nsplit;
+    int max_split;      // cap on the KV splits per head (<= kMaxSplit)
     // scratch
     float* qkv_raw;     // [3H] fp32: W_qkv ln1(x) + b_qkv, before RoPE
     half_t* attn_vec;   // [H] fp16: merged attention output (input of the O projection)
     half_t* inter;      // [F] fp16: gelu(W_up ln2(x) + b_up)
-    float* part_ml;     // [heads][nsplit][2] running max (log2 domain) and denominator
-    float* part_acc;    // [heads][nsplit][D]
+    float* part_ml;     // [heads][kMaxSplit][2] running max (log2 domain) and denominator
+    float* part_acc;    // [heads][kMaxSplit][D]
     int* head_cnt;      // [heads] arrival counters, self-resetting
-    int* bar;           // [0] epoch counter, [1] exit counter, [2] status flags
+    int* bar;           // device-wide counters, see BarSlot
+    int* mbox;          // [kMaxGrid][kMailboxInts] event flags, one line per workgroup
     // stage-C selection (split API halves)
     const half_t* c_base0;   // residual terms added to the output (nullable)
     const half_t* c_base1;
     int c_use_o, c_use_down;
+    long long* trace;   // debugging: per-workgroup phase timestamps of the fused kernel (null = off)
 };
+
+constexpr int kTraceSlots = 8;
+__device__ __forceinline__ void trace_mark(const LayerParams& p, int slot) {
+    if (p.trace != nullptr && (threadIdx.x & 63) == 0)
+        p.trace[((size_t)blockIdx.x * kMaxWaves + (threadIdx.x >> 6)) * kTraceSlots + slot] = wall_clock64();
+}
 
 // ------------------------------------------------------------------------------------------------
 // loads / conversions
@@ -89,8 +107,17 @@ __device__ __forceinline__ void st_agent(half_t* p, half_t v) {
 __device__ __forceinline__ void st_agent(uint32_t* p, uint32_t v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void st_agent2(float* p, float a, float b) {   // p 8-byte aligned
+    const uint64_t v = (uint64_t)__float_as_uint(a) | ((uint64_t)__float_as_uint(b) << 32);
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ float ld_agent(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void ld_agent2(const float* p, float& a, float& b) {   // p 8-byte aligned
+    const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    a = __uint_as_float((uint32_t)v);
+    b = __uint_as_float((uint32_t)(v >> 32));
 }
 __device__ __forceinline__ u32x4 ld_agent16(const void* p) {
     const uint64_t* q = reinterpret_cast<const uint64_t*>(p);
@@ -146,6 +173,7 @@ __device__ __forceinline__ float wave_sum(float v) {     // wave-uniform result
     return (rl(v, 0) + rl(v, 16)) + (rl(v, 32) + rl(v, 48));
 }
 __device__ __forceinline__ float xor_shfl(float v, int mask) { return __shfl_xor(v, mask, kWave); }
+__device__ __forceinline__ int first_lane(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // ------------------------------------------------------------------------------------------------
 // math
@@ -163,187 +191,290 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // ------------------------------------------------------------------------------------------------
 // device-wide synchronisation (bounded spins; a timeout raises a status flag and falls through)
 // ------------------------------------------------------------------------------------------------
-// arrive: the caller has drained its stores (and, for a workgroup-wide arrival, synchronised the workgroup)
+// Device-wide events.  Arrivals are counted in one counter per event; the wave whose arrival completes
+// the count writes a flag into one mailbox line per workgroup, and waiters poll only their own
+// workgroup's line.  (Letting every waiting wave poll the shared counter floods a single memory channel
+// with coherent loads and slows the streaming loads of the whole chip.)
+constexpr int kMailboxInts = 16;       // one 64-byte line per workgroup
+constexpr int kMaxGrid = 1024;         // workgroups a fused launch may have
+
 __device__ __forceinline__ void counter_add(int* ctr, int v) {
     __hip_atomic_fetch_add(ctr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// one thread polls; the whole workgroup leaves together.  Data published before the arrivals must be
-// read with ld_agent / ld_agent16.
-__device__ __forceinline__ void grid_wait(int* ctr, int target, int* status) {
-    if (threadIdx.x == 0) {
-        long long spins = 0;
-        while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-            __builtin_amdgcn_s_sleep(1);
-            if (++spins > kSpinLimit) {
-                __hip_atomic_fetch_or(status, kStatusSpin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                break;
-            }
+__device__ __forceinline__ int counter_peek(const int* ctr) {
+    return __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void raise_status(int* status, int flag) {
+    __hip_atomic_fetch_or(status, flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Called by a whole wave after its stores: drains them, counts the arrival, and if it is the last of
+// `target` arrivals raises mailbox slot `slot` of all `nwg` workgroups.
+__device__ __forceinline__ void event_arrive(int* ctr, int target, int* mbox, int slot, int nwg) {
+    const int lane = threadIdx.x & 63;
+    drain_memory_ops();
+    int last = 0;
+    if (lane == 0) last = (__hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == target - 1);
+    if (__builtin_amdgcn_readfirstlane(last)) {
+        for (int w = lane; w < nwg; w += kWave)
+            __hip_atomic_store(mbox + w * kMailboxInts + slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+// One lane polls this workgroup's mailbox line, the wave leaves together.  Data published before the
+// arrivals must be read with ld_agent / ld_agent16.  A wait that expires raises a status flag and
+// falls through.
+__device__ __forceinline__ void event_wait(const int* mbox, int slot, int* status) {
+    if ((threadIdx.x & 63) == 0) {
+        const int* f = mbox + blockIdx.x * kMailboxInts + slot;
+        int spins = 0;
+        while (counter_peek(f) == 0) {
+            __builtin_amdgcn_s_sleep(2);
+            if (++spins > kSpinLimit) { raise_status(status, kStatusSpin); break; }
         }
     }
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
 __device__ __forceinline__ int load_seq_len(const LayerParams& p) {
     int S = p.d_seq_len ? *p.d_seq_len : p.seq_len;
     if (S < 0 || S > p.cache_rows) {
-        if (threadIdx.x == 0 && blockIdx.x == 0)
-            __hip_atomic_fetch_or(p.bar + 2, kStatusSeq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0 && blockIdx.x == 0) raise_status(p.bar + kBarStatus, kStatusSeq);
         S = S < 0 ? 0 : p.cache_rows;
     }
     return S;
+}
+// KV splits per head for a sequence length: about kSplitRows cache rows per item
+__device__ __forceinline__ int effective_split(const LayerParams& p, int S) {
+    int n = (S + kSplitRows - 1) / kSplitRows;
+    n = n < 1 ? 1 : n;
+    return n < p.max_split ? n : p.max_split;
 }
 
 // ------------------------------------------------------------------------------------------------
 // stage A: LayerNorm into registers, then row-per-wave streaming GEMV
 // ------------------------------------------------------------------------------------------------
 // Every wave loads the whole input row (lane l holds columns i*512 + 8l .. +8 of every chunk i),
-// computes mean and variance two-pass in fp32, and keeps both affine variants (input LN for QKV,
-// post-attention LN for the MLP; they share the statistics because the residual is parallel,
-// reference include/5090/pythia_2b8/kernel.cuh:811-818) as packed fp16.
+// computes mean and variance two-pass in fp32 and keeps the normalised, affine-transformed row as
+// packed fp16.  The post-attention LayerNorm (input of the MLP) shares the statistics with the input
+// LayerNorm because the residual is parallel (reference include/5090/pythia_2b8/kernel.cuh:811-818):
+// ln_affine() re-reads x (8 KB, cache resident) with the saved statistics when that variant is needed,
+// so only one variant is live at a time.  x stays packed and is unpacked per pass (register budget).
+struct LnStats { float mean, rstd; };
+
+// Compiler-only barrier on a packed register: stops common-subexpression elimination from keeping the
+// fp32 expansion of x alive across the LayerNorm passes (it emits no instruction).
+__device__ __forceinline__ void keep_packed(u32x4& v) {
+    asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
+}
+
 template <int NCH>
-__device__ __forceinline__ void load_ln_pair(const half_t* __restrict__ x, int H, float eps,
-                                             const half_t* __restrict__ w1, const half_t* __restrict__ b1,
-                                             const half_t* __restrict__ w2, const half_t* __restrict__ b2,
-                                             int lane, half2_t (&x1)[NCH][4], half2_t (&x2)[NCH][4]) {
-    float xv[NCH][8];
-    float s = 0.f;
+__device__ __forceinline__ void ln_apply(const u32x4 (&rx)[NCH], const u32x4 (&rw)[NCH], const u32x4 (&rb)[NCH], int H,
+                                         LnStats st, int lane, half2_t (&dst)[NCH][4]) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const bool in = i * kChunk + lane * 8 < H;
+        float xv[8], g[8], b[8], y[8];
+        unpack8(rx[i], xv); unpack8(rw[i], g); unpack8(rb[i], b);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) y[j] = in ? (xv[j] - st.mean) * st.rstd * g[j] + b[j] : 0.f;
+        const u32x4 pk = pack8(y);
+        dst[i][0] = as_h2(pk.x); dst[i][1] = as_h2(pk.y); dst[i][2] = as_h2(pk.z); dst[i][3] = as_h2(pk.w);
+    }
+}
+
+template <int NCH>
+__device__ __forceinline__ void ln_load3(const half_t* __restrict__ x, const half_t* __restrict__ w,
+                                         const half_t* __restrict__ b, int H, int lane, u32x4 (&rx)[NCH],
+                                         u32x4 (&rw)[NCH], u32x4 (&rb)[NCH]) {
+    const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
         const int col = i * kChunk + lane * 8;
-        if (col < H) {
-            unpack8(ld16(x + col), xv[i]);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) s += xv[i][j];
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) xv[i][j] = 0.f;
-        }
+        const bool in = col < H;
+        rx[i] = in ? ld16(x + col) : z;
+        rw[i] = in ? ld16(w + col) : z;
+        rb[i] = in ? ld16(b + col) : z;
     }
-    const float mean = wave_sum(s) / (float)H;
+}
+
+template <int NCH>
+__device__ __forceinline__ LnStats ln_first(const half_t* __restrict__ x, int H, float eps, const half_t* __restrict__ w,
+                                            const half_t* __restrict__ b, int lane, half2_t (&dst)[NCH][4]) {
+    // x first; the affine vectors are fetched after the statistics (they are cache resident: every
+    // workgroup reads the same few KB), which keeps fewer registers live beside a prefetched weight tile
+    u32x4 rx[NCH];
+    const u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int col = i * kChunk + lane * 8;
+        rx[i] = col < H ? ld16(x + col) : z;
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        float xv[8];
+        unpack8(rx[i], xv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += xv[j];
+    }
+    LnStats st;
+    st.mean = wave_sum(s) / (float)H;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) keep_packed(rx[i]);
     float q = 0.f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
         if (i * kChunk + lane * 8 < H) {
+            float xv[8];
+            unpack8(rx[i], xv);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) { const float d = xv[i][j] - mean; q += d * d; }
+            for (int j = 0; j < 8; ++j) { const float d = xv[j] - st.mean; q += d * d; }
         }
     }
-    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)H + eps);
+    st.rstd = 1.0f / sqrtf(wave_sum(q) / (float)H + eps);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) keep_packed(rx[i]);
+    u32x4 rw[NCH], rb[NCH];
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
         const int col = i * kChunk + lane * 8;
-        float y1[8], y2[8];
-        if (col < H) {
-            float g[8], b[8];
-            unpack8(ld16(w1 + col), g); unpack8(ld16(b1 + col), b);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) y1[j] = (xv[i][j] - mean) * rstd * g[j] + b[j];
-            if (w2 != nullptr) {
-                unpack8(ld16(w2 + col), g); unpack8(ld16(b2 + col), b);
-#pragma unroll
-                for (int j = 0; j < 8; ++j) y2[j] = (xv[i][j] - mean) * rstd * g[j] + b[j];
-            } else {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) y2[j] = 0.f;
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) { y1[j] = 0.f; y2[j] = 0.f; }
-        }
-        const u32x4 p1 = pack8(y1), p2 = pack8(y2);
-        x1[i][0] = as_h2(p1.x); x1[i][1] = as_h2(p1.y); x1[i][2] = as_h2(p1.z); x1[i][3] = as_h2(p1.w);
-        x2[i][0] = as_h2(p2.x); x2[i][1] = as_h2(p2.y); x2[i][2] = as_h2(p2.z); x2[i][3] = as_h2(p2.w);
+        rw[i] = col < H ? ld16(w + col) : z;
+        rb[i] = col < H ? ld16(b + col) : z;
     }
+    ln_apply<NCH>(rx, rw, rb, H, st, lane, dst);
+    // keep later weight loads from being scheduled up into the prologue (they would only add register pressure)
+    __builtin_amdgcn_sched_barrier(0);
+    return st;
 }
 
-// Rows first, first+stride, ... < nrows of W[nrows, K]; RPI rows in flight per wave.
-// pre(row) is evaluated together with the weight loads (bias fetch); epi(row, dot, pre) is called by
-// every lane with the wave-uniform dot product.  EXACT: K == NCH*512, every lane load is in range and
-// addresses use immediate offsets; otherwise out-of-range lane loads are redirected to column 0 (their
-// activation registers are zero, so they contribute nothing).
-template <int NCH, int RPI, bool EXACT, class Pre, class Epi>
-__device__ __forceinline__ void gemv_rows(const half_t* __restrict__ W, int K, int first, int stride, int nrows,
-                                          const half2_t (&x)[NCH][4], int lane, Pre&& pre, Epi&& epi) {
+template <int NCH>
+__device__ __forceinline__ void ln_affine(const half_t* __restrict__ x, int H, LnStats st, const half_t* __restrict__ w,
+                                          const half_t* __restrict__ b, int lane, half2_t (&dst)[NCH][4]) {
+    __builtin_amdgcn_sched_barrier(0);
+    u32x4 rx[NCH], rw[NCH], rb[NCH];
+    ln_load3<NCH>(x, w, b, H, lane, rx, rw, rb);
+    ln_apply<NCH>(rx, rw, rb, H, st, lane, dst);
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// RPI weight rows of K = up to NCH*512 halfs held in registers, plus the raw bias of each row.
+template <int NCH, int RPI>
+struct RowTile {
+    u32x4 w[RPI][NCH];
+    half_t bias[RPI];
+};
+
+// Issue the loads of rows r, r+stride, ... (RPI of them; rows >= nrows repeat row r).  EXACT: K ==
+// NCH*512, every lane load is in range and addresses use immediate offsets; otherwise out-of-range
+// lane loads are redirected to column 0 (their activation registers are zero, so they add nothing).
+template <int NCH, int RPI, bool EXACT>
+__device__ __forceinline__ void load_row_tile(RowTile<NCH, RPI>& t, const half_t* __restrict__ W, int K,
+                                              const half_t* __restrict__ bias, int r, int stride, int nrows, int lane) {
     const int colb = lane * 8;
-    int coff[NCH];
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        const int c = i * kChunk + colb;
-        coff[i] = (EXACT || c < K) ? c : 0;
+    for (int j = 0; j < RPI; ++j) {
+        int rr = r + j * stride;
+        rr = rr < nrows ? rr : r;
+        const half_t* rp = W + (size_t)rr * (size_t)K;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = i * kChunk + colb;
+            t.w[j][i] = ld_stream16(rp + ((EXACT || c < K) ? c : 0));
+        }
+        t.bias[j] = bias ? bias[rr] : (half_t)0.f;
     }
-    for (int r = first; r < nrows; r += stride * RPI) {
-        u32x4 w[RPI][NCH];
-        float pv[RPI];
+}
+// epi(row, dot + bias) is called by every lane with wave-uniform arguments
+template <int NCH, int RPI, class Epi>
+__device__ __forceinline__ void finish_row_tile(const RowTile<NCH, RPI>& t, const half2_t (&x)[NCH][4], int r, int stride,
+                                                int nrows, Epi&& epi) {
 #pragma unroll
-        for (int j = 0; j < RPI; ++j) {
-            int rr = r + j * stride;
-            rr = rr < nrows ? rr : r;
-            pv[j] = pre(rr);
-            const half_t* rp = W + (size_t)rr * (size_t)K;
+    for (int j = 0; j < RPI; ++j) {
+        float acc = 0.f;
 #pragma unroll
-            for (int i = 0; i < NCH; ++i) w[j][i] = ld_stream16(EXACT ? rp + colb + i * kChunk : rp + coff[i]);
-        }
-#pragma unroll
-        for (int j = 0; j < RPI; ++j) {
-            float acc = 0.f;
-#pragma unroll
-            for (int i = 0; i < NCH; ++i) acc = dot8(w[j][i], x[i], acc);
-            acc = wave_sum(acc);
-            const int rr = r + j * stride;
-            if (rr < nrows) epi(rr, acc, pv[j]);
-        }
+        for (int i = 0; i < NCH; ++i) acc = dot8(t.w[j][i], x[i], acc);
+        acc = wave_sum(acc);
+        const int rr = r + j * stride;
+        if (rr < nrows) epi(rr, acc + (float)t.bias[j]);
     }
 }
 
-template <int NCH, class Pre, class Epi>
-__device__ __forceinline__ void gemv_rows_auto(const half_t* __restrict__ W, int K, int first, int stride, int nrows,
-                                               const half2_t (&x)[NCH][4], int lane, Pre&& pre, Epi&& epi) {
-    constexpr int RPI = (16 / NCH) > 0 ? (16 / NCH) : 1;
-    if (K == NCH * kChunk) gemv_rows<NCH, RPI, true>(W, K, first, stride, nrows, x, lane, pre, epi);
-    else gemv_rows<NCH, RPI, false>(W, K, first, stride, nrows, x, lane, pre, epi);
+// Rows first, first+stride, ... < nrows, RPI rows per tile, two tiles in flight: the loads of the next
+// tile are issued before the current one is reduced, so a wave keeps up to 2*RPI*NCH KB outstanding.
+// `pre` already holds the loads of the first tile (issued by the caller before something slow: the
+// LayerNorm prologue or a barrier).
+template <int NCH, int RPI, bool EXACT, class Epi>
+__device__ __forceinline__ void gemv_rows(const half_t* __restrict__ W, int K, const half_t* __restrict__ bias, int first,
+                                          int stride, int nrows, const half2_t (&x)[NCH][4], int lane,
+                                          RowTile<NCH, RPI>& pre, Epi&& epi) {
+    const int step = stride * RPI;
+    int r = first;
+    if (r >= nrows) return;
+    RowTile<NCH, RPI> other;
+    for (;;) {
+        const int r2 = r + step;
+        if (r2 < nrows) load_row_tile<NCH, RPI, EXACT>(other, W, K, bias, r2, stride, nrows, lane);
+        finish_row_tile<NCH, RPI>(pre, x, r, stride, nrows, epi);
+        __builtin_amdgcn_sched_barrier(0);   // a third tile's loads must not be scheduled above this point
+        if (r2 >= nrows) break;
+        r = r2 + step;
+        if (r < nrows) load_row_tile<NCH, RPI, EXACT>(pre, W, K, bias, r, stride, nrows, lane);
+        finish_row_tile<NCH, RPI>(other, x, r2, stride, nrows, epi);
+        __builtin_amdgcn_sched_barrier(0);
+        if (r >= nrows) break;
+    }
 }
 
 template <int NCH>
-__device__ __forceinline__ void stage_a_qkv(const LayerParams& p, const half2_t (&x1)[NCH][4], int gw, int nw, int lane) {
-    const half_t* __restrict__ bias = p.b_qkv;
+struct StageARpi { static constexpr int value = (16 / NCH) > 0 ? (16 / NCH) : 1; };
+
+__device__ __forceinline__ auto qkv_epilogue(const LayerParams& p, int lane) {
     float* __restrict__ dst = p.qkv_raw;
-    gemv_rows_auto<NCH>(p.w_qkv, p.H, gw, nw, 3 * p.H, x1, lane,
-                        [&](int r) { return (float)bias[r]; },
-                        [&](int r, float v, float b) { if (lane == 0) st_agent(dst + r, v + b); });
+    return [dst, lane](int r, float v) { if (lane == 0) st_agent(dst + r, v); };
 }
-template <int NCH>
-__device__ __forceinline__ void stage_a_up(const LayerParams& p, const half2_t (&x2)[NCH][4], int gw, int nw, int lane) {
-    const half_t* __restrict__ bias = p.b_up;
+__device__ __forceinline__ auto up_epilogue(const LayerParams& p, int lane) {
     half_t* __restrict__ dst = p.inter;
-    gemv_rows_auto<NCH>(p.w_up, p.H, gw, nw, p.F, x2, lane,
-                        [&](int r) { return (float)bias[r]; },
-                        [&](int r, float v, float b) { if (lane == 0) st_agent(dst + r, (half_t)gelu_tanh(v + b)); });
+    return [dst, lane](int r, float v) { if (lane == 0) st_agent(dst + r, (half_t)gelu_tanh(v)); };
 }
 
 // ------------------------------------------------------------------------------------------------
-// stage B: split-KV single-query attention for one (head, split) item, whole workgroup
+// stage B: split-KV single-query attention, one wave per (head, split) item
 // ------------------------------------------------------------------------------------------------
 // NeoX rotate-half RoPE on the first `rot` dims of a head vector held in raw fp32 scratch
 // (reference include/5090/pythia_2b8/kernel.cuh:395-421): d < rot/2 -> v[d] cos[d] - v[d+rot/2] sin[d];
 // rot/2 <= d < rot -> v[d] cos[d] + v[d-rot/2] sin[d]; d >= rot passes through.
-__device__ __forceinline__ float rope_elem(const float* __restrict__ v, int d, int rot,
-                                           const float* __restrict__ cs, const float* __restrict__ sn) {
-    const float a = ld_agent(v + d);
-    if (d >= rot) return a;
+// A lane produces dims d0 .. d0+7.  Every load (own values, rotation partners, cos, sin) is issued
+// before the first use, so the whole vector costs one memory round trip; dims >= rot use cos = 1 and
+// sin = 0 on their own value.
+__device__ __forceinline__ void rope_load8(const float* __restrict__ v, int d0, int rot, const float* __restrict__ cs,
+                                           const float* __restrict__ sn, bool act, float (&out)[8]) {
+    float a[8], pr[8], c[8], sg[8];
     const int hr = rot >> 1;
-    return d < hr ? a * cs[d] - ld_agent(v + d + hr) * sn[d] : a * cs[d] + ld_agent(v + d - hr) * sn[d];
+    if (act) {
+        ld_agent2(v + d0, a[0], a[1]); ld_agent2(v + d0 + 2, a[2], a[3]);
+        ld_agent2(v + d0 + 4, a[4], a[5]); ld_agent2(v + d0 + 6, a[6], a[7]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int d = d0 + j;
+            const bool rotd = d < rot;
+            const int pd = rotd ? (d < hr ? d + hr : d - hr) : d;
+            pr[j] = ld_agent(v + pd);
+            c[j] = rotd ? cs[d] : 1.f;
+            sg[j] = rotd ? (d < hr ? -sn[d] : sn[d]) : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) out[j] = a[j] * c[j] + pr[j] * sg[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) out[j] = 0.f;
+    }
 }
 
-struct AttnShared {
-    float m[kMaxWaves];
-    float l[kMaxWaves];
-    float acc[kMaxWaves][128];
-    int last;
-};
-
-__device__ __forceinline__ void attention_item(const LayerParams& p, int head, int sp, int S, AttnShared& sh) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+// The wave's four 16-lane groups take cache rows begin+g, begin+g+4, ...; lane `sub` of a group holds
+// dims 8 sub .. 8 sub + 7 of its row (lanes with 8 sub >= D idle).  T rows per group are in flight.
+// nwg_to_signal > 0 (fused kernel): a completed head counts towards the kBarHeads event of that many workgroups.
+__device__ __forceinline__ void attention_item(const LayerParams& p, int head, int sp, int nsplit, int S, int lane,
+                                               int nwg_to_signal) {
     const int grp = lane >> 4, sub = lane & 15;
     const int D = p.D, H = p.H, d0 = sub * 8;
     const bool act = d0 < D;
@@ -352,21 +483,19 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
     const float* __restrict__ sn = p.sin + (size_t)S * p.rope_stride;
 
     float q[8];
+    rope_load8(raw, d0, p.rot, cs, sn, act, q);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) q[j] = act ? rope_elem(raw, d0 + j, p.rot, cs, sn) * p.qscale : 0.f;
+    for (int j = 0; j < 8; ++j) q[j] *= p.qscale;
 
     float m = kNegBig, l = 0.f, acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.f;
 
     // the new token: split 0 owns it (appends it, returns it, and seeds its softmax state with it)
-    if (sp == 0 && wave == 0 && grp == 0) {
+    if (sp == 0 && grp == 0) {
         float kf[8], vf[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            kf[j] = act ? rope_elem(raw + D, d0 + j, p.rot, cs, sn) : 0.f;
-            vf[j] = act ? ld_agent(raw + 2 * D + d0 + j) : 0.f;
-        }
+        rope_load8(raw + D, d0, p.rot, cs, sn, act, kf);
+        rope_load8(raw + 2 * D, d0, 0, cs, sn, act, vf);
         const u32x4 kp = pack8(kf), vp = pack8(vf);
         unpack8(kp, kf); unpack8(vp, vf);      // attend over the fp16 values the cache will hold
         if (act) {
@@ -387,20 +516,18 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
         for (int j = 0; j < 8; ++j) acc[j] = vf[j];
     }
 
-    // cached rows of this split, interleaved over the (wave, 16-lane group) slots, 4 rows per step
-    const int chunk = (S + p.nsplit - 1) / p.nsplit;
+    const int chunk = (S + nsplit - 1) / nsplit;
     const int begin = sp * chunk;
     const int end = (begin + chunk < S) ? begin + chunk : S;
-    const int slots = nwaves * 4, slot = wave * 4 + grp;
     const half_t* __restrict__ kc = p.k_cache + (size_t)head * D + d0;
     const half_t* __restrict__ vc = p.v_cache + (size_t)head * D + d0;
-    constexpr int T = 4;
-    for (int r = begin + slot; r < end; r += slots * T) {
+    constexpr int T = 8;
+    for (int r = begin + grp; r < end; r += 4 * T) {
         u32x4 kk[T], vv[T];
         bool ok[T];
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-            const int row = r + t * slots;
+            const int row = r + t * 4;
             ok[t] = row < end;
             const u32x4 z = {0u, 0u, 0u, 0u};
             kk[t] = z; vv[t] = z;
@@ -437,7 +564,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
         m = mt;
     }
 
-    // merge the four groups of the wave (lanes sub, sub+16, sub+32, sub+48 hold the same dims)
+    // merge the four groups (lanes sub, sub+16, sub+32, sub+48 hold the same dims)
     {
         float mw = fmaxf(m, xor_shfl(m, 16));
         mw = fmaxf(mw, xor_shfl(mw, 32));
@@ -454,61 +581,67 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
         }
         m = mw;
     }
-    if (grp == 0) {
-        if (sub == 0) { sh.m[wave] = m; sh.l[wave] = l; }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) sh.acc[wave][d0 + j] = acc[j];
-    }
-    __syncthreads();
-    // merge the waves in wave order and publish the partial of this (head, split)
-    const size_t item = (size_t)head * p.nsplit + sp;
-    if ((int)threadIdx.x < D) {
-        float M = sh.m[0];
-        for (int w = 1; w < nwaves; ++w) M = fmaxf(M, sh.m[w]);
-        float L = 0.f, A = 0.f;
-        for (int w = 0; w < nwaves; ++w) {
-            const float sc = fast_exp2(sh.m[w] - M);
-            L += sh.l[w] * sc;
-            A += sh.acc[w][threadIdx.x] * sc;
-        }
-        st_agent(p.part_acc + item * D + threadIdx.x, A);
-        if (threadIdx.x == 0) { st_agent(p.part_ml + item * 2, M); st_agent(p.part_ml + item * 2 + 1, L); }
+    // publish the partial of this (head, split)
+    const size_t item = (size_t)head * kMaxSplit + sp;
+    if (grp == 0 && act) {
+        float* dst = p.part_acc + item * D + d0;
+        st_agent2(dst, acc[0], acc[1]); st_agent2(dst + 2, acc[2], acc[3]);
+        st_agent2(dst + 4, acc[4], acc[5]); st_agent2(dst + 6, acc[6], acc[7]);
+        if (sub == 0) st_agent2(p.part_ml + item * 2, m, l);
     }
     drain_memory_ops();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const int old = __hip_atomic_fetch_add(p.head_cnt + head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        sh.last = (old == p.nsplit - 1);
-    }
-    __syncthreads();
-    if (sh.last) {
-        // the last workgroup of this head merges the splits in split order; two dims per thread
-        const int t2 = threadIdx.x * 2;
-        if (t2 < D) {
-            const size_t hb = (size_t)head * p.nsplit;
-            float M = kNegBig;
-            for (int i = 0; i < p.nsplit; ++i) M = fmaxf(M, ld_agent(p.part_ml + (hb + i) * 2));
-            float L = 0.f, A0 = 0.f, A1 = 0.f;
-            for (int i = 0; i < p.nsplit; ++i) {
-                const float sc = fast_exp2(ld_agent(p.part_ml + (hb + i) * 2) - M);
-                L += ld_agent(p.part_ml + (hb + i) * 2 + 1) * sc;
-                A0 += ld_agent(p.part_acc + (hb + i) * D + t2) * sc;
-                A1 += ld_agent(p.part_acc + (hb + i) * D + t2 + 1) * sc;
+    int last = 0;
+    if (lane == 0) last = (__hip_atomic_fetch_add(p.head_cnt + head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nsplit - 1);
+    last = first_lane(last);
+    if (last) {
+        // The last wave of this head merges the splits.  Lane i fetches (m_i, l_i) of split i, so the
+        // scales come from one round trip; the accumulators (two dims per lane) are fetched eight
+        // splits at a time and added in split order.
+        const size_t hb = (size_t)head * kMaxSplit;
+        float mi = kNegBig, li = 0.f;
+        if (lane < nsplit) ld_agent2(p.part_ml + (hb + lane) * 2, mi, li);
+        float M = fmaxf(mi, xor_shfl(mi, 32));
+        M = fmaxf(M, xor_shfl(M, 16));
+        M = fmaxf(M, xor_shfl(M, 8));
+        M = fmaxf(M, xor_shfl(M, 4));
+        M = fmaxf(M, xor_shfl(M, 2));
+        M = fmaxf(M, xor_shfl(M, 1));
+        const float sci = fast_exp2(mi - M);      // scale of split `lane`
+        const float lsi = li * sci;
+        const int t2 = lane * 2;
+        const bool dact = t2 < D;
+        float L = 0.f, A0 = 0.f, A1 = 0.f;
+        for (int i0 = 0; i0 < nsplit; i0 += 8) {
+            float a0[8], a1[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                a0[u] = 0.f; a1[u] = 0.f;
+                if (dact && i0 + u < nsplit) ld_agent2(p.part_acc + (hb + i0 + u) * D + t2, a0[u], a1[u]);
             }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i = i0 + u < nsplit ? i0 + u : 0;
+                const float sc = i0 + u < nsplit ? rl(sci, i) : 0.f;
+                L += i0 + u < nsplit ? rl(lsi, i) : 0.f;
+                A0 += a0[u] * sc;
+                A1 += a1[u] * sc;
+            }
+        }
+        if (dact) {
             const half2_t o = {(half_t)(A0 / L), (half_t)(A1 / L)};
             st_agent(reinterpret_cast<uint32_t*>(p.attn_vec + (size_t)head * D + t2), as_u32(o));
         }
-        if (threadIdx.x == 0) __hip_atomic_store(p.head_cnt + head, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) __hip_atomic_store(p.head_cnt + head, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (nwg_to_signal > 0) event_arrive(p.bar + kBarHeads, p.heads, p.mbox, kBarHeads, nwg_to_signal);
     }
-    __syncthreads();   // sh is reused by the next item
 }
 
 // ------------------------------------------------------------------------------------------------
 // stage C: out[r] = base0[r] + base1[r] + bias1[r] + bias2[r] + W1[r,:] x1 + W2[r,:] x2
 // ------------------------------------------------------------------------------------------------
 struct StageC {
-    const half_t *W1, *x1, *bias1; int K1;
-    const half_t *W2, *x2, *bias2; int K2;
+    const half_t *W1, *x1, *bias1; int K1;    // O projection:  x1 = merged attention output
+    const half_t *W2, *x2, *bias2; int K2;    // MLP down:      x2 = MLP intermediate
     const half_t *base0, *base1;
     half_t* out;
     int nrows;
@@ -522,68 +655,97 @@ __device__ __forceinline__ StageC make_stage_c(const LayerParams& p) {
     return c;
 }
 
-struct StageCShared { float red[kRowBatch][kMaxWaves]; };
+constexpr int kStreamers = 4;          // streaming waves per workgroup: one per SIMD of the compute unit
+struct StageCShared { float red[kRowBatch][kStreamers]; };
 
-// The workgroup's waves form RG row groups x KS K-slices (wave = rg*KS + ks).  K is cut into
-// 512-half chunks over the concatenation [x1 | x2]; slice ks owns chunks ks, ks+KS, ... (at most CPW).
-template <int CPW>
-__device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, int KS, int RG, StageCShared& sh) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int ks = wave % KS, rg = wave / KS;
+// Stage C for the rows of workgroup `wg`: one GEMV over the concatenated input [x1 | x2].  Called by
+// every wave of the workgroup; waves >= kStreamers only take part in the workgroup barriers.
+// K is cut into 512-half chunks over the concatenation; streaming wave ks owns chunks ks, ks+4, ...
+// (at most CP), keeps its slices of x in registers, streams RPI rows per tile with two tiles in flight,
+// and leaves its partial dot product of every row in LDS; the partials are then added in wave order
+// together with the biases and residual terms: deterministic, and identical in both modes.
+// `ready()` runs after the loads of the first tile are in flight and before x is read (x is produced by
+// other workgroups; the fused kernel waits for it there, so the wait overlaps the loads).
+template <int CP, class Ready>
+__device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, StageCShared& sh, Ready&& ready) {
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int r0 = (int)(((long long)wg * c.nrows) / nwg), r1 = (int)(((long long)(wg + 1) * c.nrows) / nwg);
+    constexpr int RPI = (16 / CP) > 0 ? (16 / CP) : 1;
     const int nch1 = (c.K1 + kChunk - 1) / kChunk, nch2 = (c.K2 + kChunk - 1) / kChunk;
-    constexpr int RPI = (12 / CPW) > 0 ? (12 / CPW) : 1;
 
-    // per-chunk weight pointer at row 0; a chunk that does not exist for this lane reads a valid dummy
-    // location with row stride 0 and a zero activation slice
-    const half_t* wp[CPW];
-    int wstride[CPW];
-    half2_t xs[CPW][4];
+    // per-chunk row-0 pointer and row stride; a chunk that does not exist for this lane reads a valid
+    // dummy location with stride 0 and a zero activation slice
+    const half_t* wp[CP];
+    const half_t* xp[CP];
+    int wstride[CP];
     const half_t* dummy = c.W1 ? c.W1 : c.W2;
 #pragma unroll
-    for (int i = 0; i < CPW; ++i) {
-        const int ch = ks + i * KS;
-        wp[i] = dummy; wstride[i] = 0;
-        const half_t* xp = nullptr;
+    for (int i = 0; i < CP; ++i) {
+        const int ch = wave + i * kStreamers;
+        wp[i] = dummy; wstride[i] = 0; xp[i] = nullptr;
         if (ch < nch1) {
             const int col = ch * kChunk + lane * 8;
-            if (col < c.K1) { wp[i] = c.W1 + col; wstride[i] = c.K1; xp = c.x1 + col; }
+            if (col < c.K1) { wp[i] = c.W1 + col; wstride[i] = c.K1; xp[i] = c.x1 + col; }
         } else if (ch < nch1 + nch2) {
             const int col = (ch - nch1) * kChunk + lane * 8;
-            if (col < c.K2) { wp[i] = c.W2 + col; wstride[i] = c.K2; xp = c.x2 + col; }
+            if (col < c.K2) { wp[i] = c.W2 + col; wstride[i] = c.K2; xp[i] = c.x2 + col; }
         }
-        u32x4 xv = {0u, 0u, 0u, 0u};
-        if (xp) xv = ld_agent16(xp);
-        xs[i][0] = as_h2(xv.x); xs[i][1] = as_h2(xv.y); xs[i][2] = as_h2(xv.z); xs[i][3] = as_h2(xv.w);
     }
-
-    const int r0 = (int)(((long long)wg * c.nrows) / nwg), r1 = (int)(((long long)(wg + 1) * c.nrows) / nwg);
+    bool first = true;
+    half2_t xs[CP][4];
     for (int b0 = r0; b0 < r1; b0 += kRowBatch) {
         const int b1 = (b0 + kRowBatch < r1) ? b0 + kRowBatch : r1;
-        for (int r = b0 + rg; r < b1; r += RG * RPI) {
-            u32x4 w[RPI][CPW];
+        if (wave < kStreamers) {
+            auto load_rows = [&](u32x4 (&w)[RPI][CP], int r) {
 #pragma unroll
-            for (int j = 0; j < RPI; ++j) {
-                int rr = r + j * RG;
-                rr = rr < b1 ? rr : r;
+                for (int j = 0; j < RPI; ++j) {
+                    const int rr = (r + j < b1) ? r + j : r;
 #pragma unroll
-                for (int i = 0; i < CPW; ++i) w[j][i] = ld_stream16(wp[i] + (size_t)rr * wstride[i]);
+                    for (int i = 0; i < CP; ++i) w[j][i] = ld_stream16(wp[i] + (size_t)rr * wstride[i]);
+                }
+            };
+            auto finish_rows = [&](const u32x4 (&w)[RPI][CP], int r) {
+#pragma unroll
+                for (int j = 0; j < RPI; ++j) {
+                    float acc = 0.f;
+#pragma unroll
+                    for (int i = 0; i < CP; ++i) acc = dot8(w[j][i], xs[i], acc);
+                    acc = wave_sum(acc);
+                    if (r + j < b1 && lane == 0) sh.red[r + j - b0][wave] = acc;
+                }
+            };
+            u32x4 wa[RPI][CP], wb[RPI][CP];
+            load_rows(wa, b0);
+            if (first) {
+                ready();
+#pragma unroll
+                for (int i = 0; i < CP; ++i) {
+                    u32x4 xv = {0u, 0u, 0u, 0u};
+                    if (xp[i]) xv = ld_agent16(xp[i]);
+                    xs[i][0] = as_h2(xv.x); xs[i][1] = as_h2(xv.y); xs[i][2] = as_h2(xv.z); xs[i][3] = as_h2(xv.w);
+                }
             }
-#pragma unroll
-            for (int j = 0; j < RPI; ++j) {
-                float acc = 0.f;
-#pragma unroll
-                for (int i = 0; i < CPW; ++i) acc = dot8(w[j][i], xs[i], acc);
-                acc = wave_sum(acc);
-                const int rr = r + j * RG;
-                if (rr < b1 && lane == 0) sh.red[rr - b0][ks] = acc;
+            int r = b0;
+            for (;;) {
+                const int r2 = r + RPI;
+                if (r2 < b1) load_rows(wb, r2);
+                finish_rows(wa, r);
+                __builtin_amdgcn_sched_barrier(0);   // a third tile's loads must not be scheduled above this point
+                if (r2 >= b1) break;
+                r = r2 + RPI;
+                if (r < b1) load_rows(wa, r);
+                finish_rows(wb, r2);
+                __builtin_amdgcn_sched_barrier(0);
+                if (r >= b1) break;
             }
         }
+        first = false;
         __syncthreads();
         const int t = threadIdx.x;
         if (t < b1 - b0) {
             const int r = b0 + t;
             float v = 0.f;
-            for (int k = 0; k < KS; ++k) v += sh.red[t][k];
+            for (int k = 0; k < kStreamers; ++k) v += sh.red[t][k];
             if (c.bias1) v += (float)c.bias1[r];
             if (c.bias2) v += (float)c.bias2[r];
             if (c.base0) v += (float)c.base0[r];

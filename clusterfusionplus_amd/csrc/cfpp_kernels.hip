@@ -21,75 +21,151 @@ using namespace cfpp;
 // =================================================================================================
 namespace {
 
+// EX (hidden == NCH*512) is a template parameter of every kernel, chosen by the host: a run-time branch
+// between the two variants makes the compiler keep two copies of the in-flight tiles.
+// MLP-up rows of one wave: batches first, first+stride, ... of kUpRpi adjacent rows, two batches in flight
+template <int NCH, bool EX>
+__device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], int first, int stride, int lane) {
+    const int nbatch = (p.F + kUpRpi - 1) / kUpRpi;
+    int j = first;
+    if (j >= nbatch) return;
+    auto epi = up_epilogue(p, lane);
+    RowTile<NCH, kUpRpi> ta, tb;
+    load_row_tile<NCH, kUpRpi, EX>(ta, p.w_up, p.H, p.b_up, j * kUpRpi, 1, p.F, lane);
+    for (;;) {
+        const int j2 = j + stride;
+        if (j2 < nbatch) load_row_tile<NCH, kUpRpi, EX>(tb, p.w_up, p.H, p.b_up, j2 * kUpRpi, 1, p.F, lane);
+        finish_row_tile<NCH, kUpRpi>(ta, x2, j * kUpRpi, 1, p.F, epi);
+        __builtin_amdgcn_sched_barrier(0);
+        if (j2 >= nbatch) break;
+        j = j2 + stride;
+        if (j < nbatch) load_row_tile<NCH, kUpRpi, EX>(ta, p.w_up, p.H, p.b_up, j * kUpRpi, 1, p.F, lane);
+        finish_row_tile<NCH, kUpRpi>(tb, x2, j2 * kUpRpi, 1, p.F, epi);
+        __builtin_amdgcn_sched_barrier(0);
+        if (j >= nbatch) break;
+    }
+}
+
 // ---- split mode: one launch per stage ----------------------------------------------------------
-template <int NCH, int NWV>
-__global__ __launch_bounds__(NWV * 64) void k_stage_a(LayerParams p, int do_qkv, int do_up) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int gw = blockIdx.x * NWV + wave, nw = gridDim.x * NWV;
-    half2_t x1[NCH][4], x2[NCH][4];
-    load_ln_pair<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, lane, x1, x2);
-    if (do_qkv) stage_a_qkv<NCH>(p, x1, gw, nw, lane);
-    if (do_up) stage_a_up<NCH>(p, x2, gw, nw, lane);
+// Four waves per workgroup everywhere: one per SIMD.  A second wave on a SIMD gets far less of the
+// memory pipeline than the first while both stream, so extra streaming waves only add imbalance.
+template <int NCH, bool EX>
+__global__ __launch_bounds__(kStreamers * 64) void k_stage_a(LayerParams p) {
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
+    const int gw = blockIdx.x * kStreamers + wave, nw = gridDim.x * kStreamers;
+    constexpr int RPIA = StageARpi<NCH>::value;
+    const int nq = 3 * p.H;
+    RowTile<NCH, RPIA> t0;
+    if (gw < nq) load_row_tile<NCH, RPIA, EX>(t0, p.w_qkv, p.H, p.b_qkv, gw, nw, nq, lane);
+    half2_t xr[NCH][4];
+    const LnStats st = ln_first<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, lane, xr);
+    gemv_rows<NCH, RPIA, EX>(p.w_qkv, p.H, p.b_qkv, gw, nw, nq, xr, lane, t0, qkv_epilogue(p, lane));
+    ln_affine<NCH>(p.x, p.H, st, p.ln2_w, p.ln2_b, lane, xr);
+    up_rows<NCH, EX>(p, xr, gw, nw, lane);
 }
 
-// launched with the same workgroup size as the fused kernel so that both modes add in the same order
-__global__ __launch_bounds__(kMaxWaves * 64) void k_stage_b(LayerParams p) {
-    __shared__ AttnShared sh;
+// one (head, split) item per wave
+__global__ __launch_bounds__(kStreamers * 64) void k_stage_b(LayerParams p) {
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int S = load_seq_len(p);
-    const int nitems = p.heads * p.nsplit;
-    for (int item = blockIdx.x; item < nitems; item += gridDim.x)
-        attention_item(p, item / p.nsplit, item % p.nsplit, S, sh);
+    const int nsplit = effective_split(p, S);
+    const int item = blockIdx.x * kStreamers + wave;
+    if (item < p.heads * nsplit) attention_item(p, item / nsplit, item % nsplit, nsplit, S, lane, 0);
 }
 
-template <int CPW, int NWV>
-__global__ __launch_bounds__(NWV * 64) void k_stage_c(LayerParams p, int KS, int RG) {
+template <int CPC>
+__global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
     __shared__ StageCShared sh;
     const StageC c = make_stage_c(p);
-    stage_c_rows<CPW>(c, blockIdx.x, gridDim.x, KS, RG, sh);
+    stage_c_rows<CPC>(c, blockIdx.x, gridDim.x, sh, [] {});
 }
 
 // ---- fused mode: one persistent launch ---------------------------------------------------------
-// Timeline of every workgroup (NW = total waves in the grid):
-//   LN -> QKV rows -> [arrive, per wave] -> MLP-up rows -> wait(epoch 1: all QKV rows written;
-//   the wait is hidden behind the MLP-up rows) -> attention items -> [arrive] -> wait(epoch 2)
-//   -> stage C rows -> exit counter (the last workgroup resets the counters for the next launch).
-// All workgroups must be co-resident: the host launches at most one per compute unit.
-template <int NCH, int CPW, int NWV>
-__global__ __launch_bounds__(NWV * 64) void k_fused(LayerParams p, int KS, int RG) {
-    __shared__ AttnShared sha;
+// One workgroup per compute unit, eight waves: four streaming waves (one per SIMD) and four helper waves.
+//   streaming wave: first QKV tile in flight -> LayerNorm -> its QKV rows -> bump kBarQkv -> its MLP-up
+//                   rows -> bump kBarUp -> (helps with attention items if any are left) -> stage C: first
+//                   weight tile in flight, wait for kBarUp and kBarHeads, O-projection + MLP-down rows,
+//                   row reduction, bias, residual.
+//   helper wave:    waits for kBarQkv, then takes (head, split) attention items from the workgroup's
+//                   queue at raised wave priority.  Attention is a chain of dependent memory round
+//                   trips; it runs beside the MLP-up streaming instead of in front of it.
+// The last workgroup to leave zeroes the counters for the next launch.  All workgroups must be
+// co-resident (the host launches one per compute unit); every wait is bounded.
+struct FusedShared { int attn_next; };
+
+__device__ __forceinline__ int lds_take(int* p) { return __hip_atomic_fetch_add(p, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+
+template <int NCH, int CPC, bool EX>
+__global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
+    __shared__ FusedShared q;
     __shared__ StageCShared shc;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int G = gridDim.x, gw = blockIdx.x * NWV + wave, nw = G * NWV;
-    int* epoch = p.bar;
-    int* exitc = p.bar + 1;
-    int* status = p.bar + 2;
-    const int S = load_seq_len(p);
-    {
-        half2_t x1[NCH][4], x2[NCH][4];
-        load_ln_pair<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, lane, x1, x2);
-        stage_a_qkv<NCH>(p, x1, gw, nw, lane);
-        drain_memory_ops();
-        if (lane == 0) counter_add(epoch, 1);
-        stage_a_up<NCH>(p, x2, gw, nw, lane);
-    }
-    grid_wait(epoch, nw, status);
-    const int nitems = p.heads * p.nsplit;
-    for (int item = blockIdx.x; item < nitems; item += G)
-        attention_item(p, item / p.nsplit, item % p.nsplit, S, sha);
-    drain_memory_ops();
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
+    const int G = gridDim.x, b = blockIdx.x;
+    const int nsw = G * kStreamers;                 // streaming waves in the grid
+    int* status = p.bar + kBarStatus;
+    if (threadIdx.x == 0) q.attn_next = 0;
     __syncthreads();
-    if (threadIdx.x == 0) counter_add(epoch, NWV);
-    grid_wait(epoch, 2 * nw, status);
+    trace_mark(p, 0);
+
+    const int S = load_seq_len(p);
+    const int nsplit = effective_split(p, S);
+    const int nitems = p.heads * nsplit;
+    const int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
+    auto take_attention_items = [&] {
+        for (;;) {
+            int t = 0;
+            if (lane == 0) t = lds_take(&q.attn_next);
+            t = first_lane(t);
+            if (t >= attn_count) break;
+            const int item = b + t * G;
+            trace_mark(p, 3);
+            attention_item(p, item / nsplit, item % nsplit, nsplit, S, lane, G);
+            trace_mark(p, 4);
+        }
+    };
+
+    if (wave < kStreamers) {
+        const int sgw = b * kStreamers + wave;
+        constexpr int RPIA = StageARpi<NCH>::value;
+        const int nq = 3 * p.H;
+        half2_t xr[NCH][4];   // ln1(x) for the QKV rows, then ln2(x) for the MLP-up rows
+        RowTile<NCH, RPIA> t0;
+        if (sgw < nq) load_row_tile<NCH, RPIA, EX>(t0, p.w_qkv, p.H, p.b_qkv, sgw, nsw, nq, lane);
+        const LnStats st = ln_first<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, lane, xr);
+        trace_mark(p, 1);
+        gemv_rows<NCH, RPIA, EX>(p.w_qkv, p.H, p.b_qkv, sgw, nsw, nq, xr, lane, t0, qkv_epilogue(p, lane));
+        event_arrive(p.bar + kBarQkv, nsw, p.mbox, kBarQkv, G);
+        trace_mark(p, 2);
+        ln_affine<NCH>(p.x, p.H, st, p.ln2_w, p.ln2_b, lane, xr);
+        up_rows<NCH, EX>(p, xr, sgw, nsw, lane);
+        event_arrive(p.bar + kBarUp, nsw, p.mbox, kBarUp, G);
+        trace_mark(p, 5);
+        event_wait(p.mbox, kBarQkv, status);
+        take_attention_items();
+    } else {
+        event_wait(p.mbox, kBarQkv, status);
+        __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
+        take_attention_items();
+        __builtin_amdgcn_s_setprio(0);
+    }
     {
         const StageC c = make_stage_c(p);
-        stage_c_rows<CPW>(c, blockIdx.x, G, KS, RG, shc);
+        stage_c_rows<CPC>(c, b, G, shc, [&] {
+            event_wait(p.mbox, kBarUp, status);
+            trace_mark(p, 6);
+            event_wait(p.mbox, kBarHeads, status);
+            trace_mark(p, 7);
+        });
     }
-    if (threadIdx.x == 0) {
-        const int old = __hip_atomic_fetch_add(exitc, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (old == G - 1) {
-            __hip_atomic_store(epoch, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(exitc, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+    // the last workgroup to leave re-arms the counters and mailboxes for the next launch
+    __shared__ int last_out;
+    if (threadIdx.x == 0)
+        last_out = (__hip_atomic_fetch_add(p.bar + kBarExit, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == G - 1);
+    __syncthreads();
+    if (last_out) {
+        for (int i = threadIdx.x; i < G * kMailboxInts; i += blockDim.x)
+            __hip_atomic_store(p.mbox + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x <= kBarExit) __hip_atomic_store(p.bar + threadIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -104,24 +180,27 @@ __global__ void k_embed(const half_t* __restrict__ embed, const int* __restrict_
 }
 
 // logits = W LN(x); every workgroup also records its best (value, index) for the greedy pick
-template <int NCH, int NWV>
-__global__ __launch_bounds__(NWV * 64) void k_lm_head(const half_t* __restrict__ x, int H, float eps,
+template <int NCH, bool EX>
+__global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __restrict__ x, int H, float eps,
                                                       const half_t* __restrict__ ln_w, const half_t* __restrict__ ln_b,
                                                       const half_t* __restrict__ W, int vocab, float* __restrict__ logits,
                                                       float* __restrict__ best_val, int* __restrict__ best_idx) {
+    constexpr int NWV = kStreamers;
     __shared__ float sv[NWV];
     __shared__ int si[NWV];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int gw = blockIdx.x * NWV + wave, nw = gridDim.x * NWV;
-    half2_t x1[NCH][4], x2[NCH][4];
-    load_ln_pair<NCH>(x, H, eps, ln_w, ln_b, nullptr, nullptr, lane, x1, x2);
+    constexpr int RPIA = StageARpi<NCH>::value;
+    RowTile<NCH, RPIA> t0;
+    if (gw < vocab) load_row_tile<NCH, RPIA, EX>(t0, W, H, nullptr, gw, nw, vocab, lane);
+    half2_t x1[NCH][4];
+    ln_first<NCH>(x, H, eps, ln_w, ln_b, lane, x1);
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    gemv_rows_auto<NCH>(W, H, gw, nw, vocab, x1, lane, [&](int) { return 0.f; },
-                        [&](int r, float v, float) {
-                            if (lane == 0) logits[r] = v;
-                            if (v > bv || (v == bv && r < bi)) { bv = v; bi = r; }
-                        });
+    gemv_rows<NCH, RPIA, EX>(W, H, nullptr, gw, nw, vocab, x1, lane, t0, [&](int r, float v) {
+        if (lane == 0) logits[r] = v;
+        if (v > bv || (v == bv && r < bi)) { bv = v; bi = r; }
+    });
     if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -199,8 +278,10 @@ int env_int(const char* name, int dflt) {
 
 constexpr size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+long long* g_trace = nullptr;   // see cfpp_debug_set_trace
+
 struct WorkspaceLayout {
-    size_t qkv_raw, attn_vec, inter, part_ml, part_acc, head_cnt, bar, total;
+    size_t qkv_raw, attn_vec, inter, part_ml, part_acc, head_cnt, bar, mbox, total;
 };
 
 WorkspaceLayout workspace_layout(const cfpp_neox_dims& d) {
@@ -214,6 +295,7 @@ WorkspaceLayout workspace_layout(const cfpp_neox_dims& d) {
     w.part_acc = take((size_t)d.heads * kMaxSplit * d.head_dim * 4);
     w.head_cnt = take((size_t)d.heads * 4);
     w.bar = take(64);
+    w.mbox = take((size_t)kMaxGrid * kMailboxInts * 4);
     w.total = off;
     return w;
 }
@@ -231,22 +313,15 @@ int check_dims(const cfpp_neox_dims* d) {
 
 // launch geometry for one set of dims
 struct Plan {
-    int nch;        // 512-half chunks of the hidden row (stage A registers)
-    int nwv;        // waves per workgroup
-    int ks, rg;     // stage C: K slices x row groups = nwv
-    int cpw;        // stage C chunks per wave
+    int nch;        // 512-half chunks of the hidden row (stage-A registers)
+    int cpc;        // stage-C chunks ([attention | MLP intermediate]) per streaming wave
 };
 
 int make_plan(const cfpp_neox_dims& d, Plan* out) {
     Plan p{};
     p.nch = (d.hidden + kChunk - 1) / kChunk;
-    const int nchc = p.nch + (d.ffn + kChunk - 1) / kChunk;
-    if (p.nch == 5 && nchc == 25) { p.nwv = 10; p.ks = 5; p.rg = 2; p.cpw = 5; }   // Pythia-2.8B
-    else {
-        p.nwv = 8; p.ks = 8; p.rg = 1;
-        p.cpw = (nchc + p.ks - 1) / p.ks;
-    }
-    if (p.cpw > 8) return CFPP_ERR_DIMS;
+    p.cpc = (p.nch + (d.ffn + kChunk - 1) / kChunk + kStreamers - 1) / kStreamers;
+    if (p.nch < 1 || p.nch > 8 || p.cpc < 1 || p.cpc > 10) return CFPP_ERR_DIMS;
     *out = p;
     return CFPP_OK;
 }
@@ -263,79 +338,66 @@ int launch_check() {
 }
 
 // ---- template dispatch ---------------------------------------------------------------------------
-template <int NCH, int NWV>
-int launch_stage_a_t(const LayerParams& p, int grid, int do_qkv, int do_up, hipStream_t st) {
-    hipLaunchKernelGGL((k_stage_a<NCH, NWV>), dim3(grid), dim3(NWV * 64), 0, st, p, do_qkv, do_up);
+template <int NCH>
+int launch_stage_a_t(const LayerParams& p, int grid, hipStream_t st) {
+    if (p.H == NCH * kChunk) hipLaunchKernelGGL((k_stage_a<NCH, true>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
+    else hipLaunchKernelGGL((k_stage_a<NCH, false>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
     return launch_check();
 }
-template <int CPW, int NWV>
-int launch_stage_c_t(const LayerParams& p, int grid, int KS, int RG, hipStream_t st) {
-    hipLaunchKernelGGL((k_stage_c<CPW, NWV>), dim3(grid), dim3(NWV * 64), 0, st, p, KS, RG);
+template <int CPC>
+int launch_stage_c_t(const LayerParams& p, int grid, hipStream_t st) {
+    hipLaunchKernelGGL((k_stage_c<CPC>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
     return launch_check();
 }
-template <int NCH, int CPW, int NWV>
-int launch_fused_t(const LayerParams& p, int grid, int KS, int RG, hipStream_t st) {
+template <int NCH, int CPC>
+int launch_fused_t(const LayerParams& p, int grid, hipStream_t st) {
+    const void* fn = p.H == NCH * kChunk ? (const void*)(k_fused<NCH, CPC, true>) : (const void*)(k_fused<NCH, CPC, false>);
     static int coop = env_int("CFPP_COOPERATIVE", 0);
-    if (coop) {
-        LayerParams pp = p;
-        void* args[] = {&pp, &KS, &RG};
-        CFPP_HIP(hipLaunchCooperativeKernel((const void*)(k_fused<NCH, CPW, NWV>), dim3(grid), dim3(NWV * 64), args, 0, st));
-        return CFPP_OK;
-    }
-    hipLaunchKernelGGL((k_fused<NCH, CPW, NWV>), dim3(grid), dim3(NWV * 64), 0, st, p, KS, RG);
-    return launch_check();
-}
-template <int NCH, int CPW, int NWV>
-int fused_max_blocks_per_cu() {
-    int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)(k_fused<NCH, CPW, NWV>), NWV * 64, 0) != hipSuccess) return 0;
-    return n;
+    LayerParams pp = p;
+    void* args[] = {&pp};
+    if (coop) CFPP_HIP(hipLaunchCooperativeKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st));
+    else CFPP_HIP(hipLaunchKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st));
+    return CFPP_OK;
 }
 
 #define CFPP_NCH_CASES(X) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8)
+// (hidden chunks, stage-C chunks per streaming wave) of the Pythia family, ffn = 4 hidden:
+// 512 -> (1,2), 768/1024 -> (2,3), 2048 -> (4,5), 2560 -> (5,7), 4096 -> (8,10); (8,8) is 4096 with ffn 11008
+#define CFPP_SHAPE_CASES(X) X(1, 2) X(2, 3) X(4, 5) X(5, 7) X(8, 10) X(8, 8)
 
-int launch_stage_a(const Plan& pl, const LayerParams& p, int grid, int do_qkv, int do_up, hipStream_t st) {
-    if (pl.nwv == 10 && pl.nch == 5) return launch_stage_a_t<5, 10>(p, grid, do_qkv, do_up, st);
+int launch_stage_a(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
     switch (pl.nch) {
-#define X(n) case n: return launch_stage_a_t<n, 8>(p, grid, do_qkv, do_up, st);
+#define X(n) case n: return launch_stage_a_t<n>(p, grid, st);
         CFPP_NCH_CASES(X)
 #undef X
     }
     return CFPP_ERR_DIMS;
 }
 int launch_stage_c(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
-    if (pl.nwv == 10) return launch_stage_c_t<5, 10>(p, grid, pl.ks, pl.rg, st);
-    switch (pl.cpw) {
-#define X(n) case n: return launch_stage_c_t<n, 8>(p, grid, pl.ks, pl.rg, st);
-        CFPP_NCH_CASES(X)
+#define X(a, b) if (pl.nch == a && pl.cpc == b) return launch_stage_c_t<b>(p, grid, st);
+    CFPP_SHAPE_CASES(X)
 #undef X
-    }
     return CFPP_ERR_DIMS;
 }
-// fused kernels are instantiated for the shapes that occur in the Pythia family
-#define CFPP_FUSED_CASES(X) X(1, 1, 8) X(2, 1, 8) X(2, 2, 8) X(4, 3, 8) X(5, 5, 10) X(8, 5, 8) X(8, 4, 8)
 int launch_fused(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
-#define X(a, b, c) if (pl.nch == a && pl.cpw == b && pl.nwv == c) return launch_fused_t<a, b, c>(p, grid, pl.ks, pl.rg, st);
-    CFPP_FUSED_CASES(X)
+#define X(a, b) if (pl.nch == a && pl.cpc == b) return launch_fused_t<a, b>(p, grid, st);
+    CFPP_SHAPE_CASES(X)
 #undef X
     return CFPP_ERR_DIMS;
 }
-bool fused_available(const Plan& pl) {
-#define X(a, b, c) if (pl.nch == a && pl.cpw == b && pl.nwv == c) return fused_max_blocks_per_cu<a, b, c>() >= 1;
-    CFPP_FUSED_CASES(X)
+bool shape_supported(const Plan& pl) {
+#define X(a, b) if (pl.nch == a && pl.cpc == b) return true;
+    CFPP_SHAPE_CASES(X)
 #undef X
     return false;
 }
 
-int choose_nsplit(const cfpp_neox_dims& d, int seq_hint, int cus) {
-    // enough (head, split) items to cover the chip, at least ~64 cache rows per item
-    int by_len = (seq_hint + 63) / 64;
-    int by_chip = (cus + d.heads - 1) / d.heads;
-    int n = by_len < by_chip ? by_len : by_chip;
-    n = env_int("CFPP_NSPLIT", n);
-    if (n < 1) n = 1;
-    if (n > kMaxSplit) n = kMaxSplit;
-    return n;
+// upper bound of the KV splits per head the kernels will use for a sequence length (device code
+// computes the same value from the actual length: effective_split)
+int split_bound(int seq_hint, int max_split) {
+    int n = (seq_hint + kSplitRows - 1) / kSplitRows;
+    n = n < 1 ? 1 : n;
+    return n < max_split ? n : max_split;
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -360,6 +422,7 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     if (ws_bytes < L.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CFPP_ERR_WORKSPACE;
     rc = make_plan(*d, plan);
     if (rc) return rc;
+    if (!shape_supported(*plan)) return CFPP_ERR_DIMS;
 
     LayerParams p{};
     p.H = d->hidden; p.heads = d->heads; p.D = d->head_dim; p.rot = d->rotary_dim; p.F = d->ffn;
@@ -375,8 +438,9 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     p.cache_rows = io->cache_rows;
     p.cos = io->cos; p.sin = io->sin; p.rope_stride = io->rope_stride;
     p.seq_len = io->seq_len; p.d_seq_len = io->d_seq_len;
-    int hint = io->d_seq_len ? (io->max_seq_len > 0 ? io->max_seq_len : io->cache_rows) : io->seq_len;
-    p.nsplit = choose_nsplit(*d, hint, device_info().cus);
+    p.max_split = env_int("CFPP_MAX_SPLIT", kMaxSplit);
+    if (p.max_split < 1) p.max_split = 1;
+    if (p.max_split > kMaxSplit) p.max_split = kMaxSplit;
     char* ws = reinterpret_cast<char*>(workspace);
     p.qkv_raw = reinterpret_cast<float*>(ws + L.qkv_raw);
     p.attn_vec = reinterpret_cast<half_t*>(ws + L.attn_vec);
@@ -385,9 +449,15 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     p.part_acc = reinterpret_cast<float*>(ws + L.part_acc);
     p.head_cnt = reinterpret_cast<int*>(ws + L.head_cnt);
     p.bar = reinterpret_cast<int*>(ws + L.bar);
+    p.mbox = reinterpret_cast<int*>(ws + L.mbox);
     p.c_base0 = p.x; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 1;
+    p.trace = g_trace;
     *out = p;
     return CFPP_OK;
+}
+
+int seq_hint_of(const cfpp_neox_io* io) {
+    return io->d_seq_len ? (io->max_seq_len > 0 ? io->max_seq_len : io->cache_rows) : io->seq_len;
 }
 
 int grid_for_streaming(const Plan&) {
@@ -396,14 +466,13 @@ int grid_for_streaming(const Plan&) {
     return cus * env_int("CFPP_WG_PER_CU", 1);
 }
 
-int run_split(const Plan& pl, LayerParams& p, bool full_layer, hipStream_t st) {
+int run_split(const Plan& pl, LayerParams& p, int seq_hint, hipStream_t st) {
     const int grid = grid_for_streaming(pl);
-    int rc = launch_stage_a(pl, p, grid, 1, 1, st);
+    int rc = launch_stage_a(pl, p, grid, st);
     if (rc) return rc;
-    int bgrid = p.heads * p.nsplit;
-    hipLaunchKernelGGL(k_stage_b, dim3(bgrid), dim3(pl.nwv * 64), 0, st, p);
+    const int bgrid = (p.heads * split_bound(seq_hint, p.max_split) + kStreamers - 1) / kStreamers;
+    hipLaunchKernelGGL(k_stage_b, dim3(bgrid), dim3(kStreamers * 64), 0, st, p);
     if ((rc = launch_check())) return rc;
-    (void)full_layer;
     return launch_stage_c(pl, p, grid, st);
 }
 
@@ -446,10 +515,10 @@ int cfpp_neox_layer_decode(const cfpp_neox_dims* dims, const cfpp_neox_weights* 
     int rc = fill_params(dims, w, io, workspace, workspace_bytes, true, true, &p, &pl);
     if (rc) return rc;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    if (mode == CFPP_MODE_SPLIT) return run_split(pl, p, true, st);
-    if (!fused_available(pl)) return CFPP_ERR_DIMS;
+    if (mode == CFPP_MODE_SPLIT) return run_split(pl, p, seq_hint_of(io), st);
     DeviceInfo& di = device_info();
-    const int grid = di.cus > 0 ? di.cus : 256;
+    int grid = di.cus > 0 ? di.cus : 256;
+    if (grid > kMaxGrid) grid = kMaxGrid;
     return launch_fused(pl, p, grid, st);
 }
 
@@ -463,7 +532,7 @@ int cfpp_neox_attention_mlp_up(const cfpp_neox_dims* dims, const cfpp_neox_weigh
     p.inter = reinterpret_cast<half_t*>(io->mlp_intermediate);   // MLP-up writes the caller's tensor directly
     p.out = reinterpret_cast<half_t*>(io->attn_output);          // stage C: W_o attn + b_o only
     p.c_base0 = nullptr; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 0;
-    return run_split(pl, p, false, reinterpret_cast<hipStream_t>(stream));
+    return run_split(pl, p, seq_hint_of(io), reinterpret_cast<hipStream_t>(stream));
 }
 
 int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void* attn_output,
@@ -479,6 +548,7 @@ int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void
     (void)workspace; (void)workspace_bytes;
     Plan pl;
     if ((rc = make_plan(*dims, &pl))) return rc;
+    if (!shape_supported(pl)) return CFPP_ERR_DIMS;
     LayerParams p{};
     p.H = dims->hidden; p.heads = dims->heads; p.D = dims->head_dim; p.rot = dims->rotary_dim; p.F = dims->ffn;
     p.w_down = reinterpret_cast<const half_t*>(w_down); p.b_down = reinterpret_cast<const half_t*>(b_down);
@@ -496,15 +566,22 @@ int cfpp_workspace_check(const cfpp_neox_dims* dims, void* workspace, void* stre
     const WorkspaceLayout L = workspace_layout(*dims);
     int* bar = reinterpret_cast<int*>(reinterpret_cast<char*>(workspace) + L.bar);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    int host[3] = {0, 0, 0};
+    int host[kBarStatus + 1] = {0};
     CFPP_HIP(hipMemcpyAsync(host, bar, sizeof(host), hipMemcpyDeviceToHost, st));
     CFPP_HIP(hipStreamSynchronize(st));
-    if (host[2] != 0 || host[0] != 0 || host[1] != 0) {
+    bool bad = false;
+    for (int i = 0; i <= kBarStatus; ++i) bad = bad || host[i] != 0;
+    if (bad) {
         // a raised flag (or counters left mid-flight by an expired wait): clear so the workspace is reusable
         CFPP_HIP(hipMemsetAsync(workspace, 0, L.total, st));
         CFPP_HIP(hipStreamSynchronize(st));
         return CFPP_ERR_DEVICE;
     }
+    return CFPP_OK;
+}
+
+int cfpp_debug_set_trace(void* device_buffer) {
+    g_trace = reinterpret_cast<long long*>(device_buffer);
     return CFPP_OK;
 }
 
@@ -609,8 +686,12 @@ int launch_lm_head(int H, int vocab, float eps, const void* x, const void* ln_w,
     switch (nch) {
 #define X(n)                                                                                                    \
     case n:                                                                                                     \
-        hipLaunchKernelGGL((k_lm_head<n, 8>), dim3(grid), dim3(512), 0, st, h(x), H, eps, h(ln_w), h(ln_b), h(W), \
-                           vocab, logits, best_val, best_idx);                                                  \
+        if (H == n * kChunk)                                                                                    \
+            hipLaunchKernelGGL((k_lm_head<n, true>), dim3(grid), dim3(kStreamers * 64), 0, st, h(x), H, eps, h(ln_w),  \
+                               h(ln_b), h(W), vocab, logits, best_val, best_idx);                               \
+        else                                                                                                    \
+            hipLaunchKernelGGL((k_lm_head<n, false>), dim3(grid), dim3(kStreamers * 64), 0, st, h(x), H, eps, h(ln_w), \
+                               h(ln_b), h(W), vocab, logits, best_val, best_idx);                               \
         return launch_check();
         CFPP_NCH_CASES(X)
 #undef X

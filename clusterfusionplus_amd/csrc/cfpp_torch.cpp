@@ -396,6 +396,16 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     DEFINE_MODEL_OPS(m, pythia_6b9)
 
     m.def("cfpp_version", []() { return std::string(cfpp_version()); });
+    m.def("debug_set_trace", [](c10::optional<Tensor> buf) {
+        // int64 device tensor of at least 1024*16*8 elements, or None to switch tracing off
+        if (buf.has_value()) {
+            TORCH_CHECK(buf->is_cuda() && buf->scalar_type() == torch::kInt64 && buf->is_contiguous() && buf->numel() >= 1024 * 16 * 8,
+                        "trace buffer must be a contiguous int64 GPU tensor with >= 131072 elements");
+            cfpp_debug_set_trace(buf->data_ptr());
+        } else {
+            cfpp_debug_set_trace(nullptr);
+        }
+    });
     m.def("workspace_bytes", [](int64_t hidden, int64_t heads, int64_t head_dim, int64_t rotary_dim, int64_t ffn) {
         cfpp_neox_dims d{(int32_t)hidden, (int32_t)heads, (int32_t)head_dim, (int32_t)rotary_dim, (int32_t)ffn, 1e-5f};
         return (int64_t)cfpp_neox_workspace_bytes(&d);

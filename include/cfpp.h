@@ -145,6 +145,11 @@ int cfpp_ctx_destroy(int family, int64_t id);
  * Returns CFPP_OK or CFPP_ERR_DEVICE.  For tests and debugging; not on the hot path. */
 int cfpp_workspace_check(const cfpp_neox_dims* dims, void* workspace, void* stream);
 
+/* Debugging aid: when set to a device buffer of cfpp_debug_trace_bytes() bytes, every fused launch
+ * stores 100 MHz timestamps of its phase boundaries per workgroup and wave
+ * ([workgroup][16 waves][8 slots] int64); NULL switches it off.  No counterpart in the reference. */
+int cfpp_debug_set_trace(void* device_buffer);
+
 /* ---- whole-model greedy decode (our counterpart of the reference's Python decode loop,
  * tests/benchmark_decode.py:147-189: embedding row -> layers -> final LayerNorm -> LM head ->
  * argmax), captured once into a hipGraph and replayed per token ------------------------------- */
