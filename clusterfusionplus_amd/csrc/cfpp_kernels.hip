@@ -832,7 +832,7 @@ int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream) {
     if (n_steps < 0) return CFPP_ERR_DIMS;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (!st) {
-        if (!s->own_stream) CFPP_HIP(hipStreamCreateWithFlags(&s->own_stream, hipStreamNonBlocking));
+        if (!s->own_stream) CFPP_HIP(hipStreamCreateWithFlags(&s->own_stream, hipStreamDefault));   // ordered with the null stream
         st = s->own_stream;
     }
     if (!s->exec) {

@@ -1,0 +1,102 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every symbol the header declares,
+and rejects bad arguments with its documented status codes before anything is launched."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "clusterfusionplus_amd", "libcfpp.so")
+HEADER = os.path.join(ROOT, "include", "cfpp.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import torch  # noqa: F401  the HIP runtime the library binds to
+    if not os.path.exists(LIB):
+        pytest.fail("libcfpp.so is not built: run `python -m clusterfusionplus_amd.build`")
+    return ctypes.CDLL(LIB)
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cfpp_[a-z0-9_]+)\s*\(", text)))
+
+
+class Dims(ctypes.Structure):
+    _fields_ = [("hidden", ctypes.c_int32), ("heads", ctypes.c_int32), ("head_dim", ctypes.c_int32),
+                ("rotary_dim", ctypes.c_int32), ("ffn", ctypes.c_int32), ("eps", ctypes.c_float)]
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = declared_functions()
+    assert len(names) >= 18, names
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, f"declared in cfpp.h but not exported by libcfpp.so: {missing}"
+
+
+def test_status_strings_and_version(lib):
+    lib.cfpp_status_str.restype = ctypes.c_char_p
+    lib.cfpp_version.restype = ctypes.c_char_p
+    assert lib.cfpp_status_str(0) == b"ok"
+    seen = {lib.cfpp_status_str(-i) for i in range(1, 9)}
+    assert len(seen) == 8 and b"unknown status" not in seen
+    assert b"gfx950" in lib.cfpp_version()
+
+
+def test_workspace_bytes_and_dims_validation(lib):
+    lib.cfpp_neox_workspace_bytes.restype = ctypes.c_size_t
+    ok = [Dims(2560, 32, 80, 20, 10240, 1e-5), Dims(4096, 32, 128, 32, 16384, 1e-5)]
+    for d in ok:
+        n = lib.cfpp_neox_workspace_bytes(ctypes.byref(d))
+        assert n > 0 and n % 256 == 0
+    bad = [Dims(2560, 32, 81, 20, 10240, 1e-5),     # hidden != heads * head_dim
+           Dims(4100, 32, 128, 32, 16384, 1e-5),
+           Dims(8192, 32, 256, 32, 32768, 1e-5),    # head_dim > 128
+           Dims(4096, 32, 128, 33, 16384, 1e-5),    # odd rotary_dim
+           Dims(4096, 32, 128, 32, 16384, 0.0)]     # eps
+    for d in bad:
+        assert lib.cfpp_neox_workspace_bytes(ctypes.byref(d)) == 0
+    assert lib.cfpp_neox_workspace_bytes(None) == 0
+
+
+def test_null_and_mode_errors_launch_nothing(lib):
+    d = Dims(4096, 32, 128, 32, 16384, 1e-5)
+    # unknown mode, NULL structs: rejected before any HIP call, so this runs without a GPU
+    assert lib.cfpp_neox_layer_decode(ctypes.byref(d), None, None, 7, None, ctypes.c_size_t(0), None) == -6
+    assert lib.cfpp_neox_layer_decode(ctypes.byref(d), None, None, 0, None, ctypes.c_size_t(0), None) == -1
+    assert lib.cfpp_neox_layer_decode(None, None, None, 0, None, ctypes.c_size_t(0), None) == -1
+    assert lib.cfpp_neox_mlp_down(ctypes.byref(d), None, None, None, None, None, None, None, ctypes.c_size_t(0), None) == -1
+    assert lib.cfpp_ctx_step(0, ctypes.c_int64(12345), None, None, 0, None, None) == -1
+    assert lib.cfpp_ctx_destroy(0, ctypes.c_int64(12345)) == 0          # unknown id: no-op
+    assert lib.cfpp_stack_create(None, None) == -1
+    assert lib.cfpp_stack_destroy(None) == 0
+    assert lib.cfpp_neox_lm_head(4096, 100, ctypes.c_float(1e-5), None, None, None, None, None, None) == -1
+
+
+def test_package_imports_and_exposes_reference_names():
+    import clusterfusion
+    want = ["pythia_2b8_decoder_layer", "pythia_2b8_decoder_layer_split", "pythia_2b8_attention_only",
+            "pythia_2b8_mlp_only", "pythia_2b8_create_graph_context", "pythia_2b8_graph_decode_step",
+            "pythia_2b8_destroy_graph_context", "pythia_6b9_decoder_layer", "pythia_6b9_create_graph_context",
+            "pythia_6b9_graph_decode_step", "pythia_6b9_destroy_graph_context"]   # reference include/pybind.cpp:284-297
+    for n in want:
+        assert callable(getattr(clusterfusion, n)), n
+    # CPU tensors are refused with an exception, not a crash
+    import torch
+    t = torch.zeros(1, 2560, dtype=torch.float16)
+    with pytest.raises(RuntimeError):
+        clusterfusion.pythia_2b8_mlp_only(t, t, t, t, t)
+    with pytest.raises(RuntimeError, match="not initialized"):
+        clusterfusion.pythia_2b8_graph_decode_step(99, t, t, t, t, t, t, t, t, t, t, t, t, t, 0)
+
+
+def test_rope_tables_match_oracle():
+    from clusterfusionplus_amd.model import rope_tables
+    from oracle.neox_oracle import rope_table
+    import torch
+    c, s = rope_tables(300, 20, device="cpu")
+    c2, s2 = rope_table(torch.arange(300), 20)
+    assert torch.equal(c, c2) and torch.equal(s, s2)
