@@ -735,6 +735,22 @@ struct cfpp_neox_stack {
 };
 
 namespace {
+int stack_enqueue_layer(cfpp_neox_stack* s, int l, hipStream_t st) {
+    const cfpp_neox_dims& d = s->desc.dims;
+    cfpp_neox_io io{};
+    io.input = s->hidden[l & 1];
+    io.output = s->hidden[(l + 1) & 1];
+    io.k_new = s->k_new; io.v_new = s->v_new;
+    io.k_cache = s->kc[l]; io.v_cache = s->vc[l];
+    io.cache_rows = s->desc.cache_rows;
+    io.cos = s->desc.rope_cos; io.sin = s->desc.rope_sin;
+    io.rope_stride = d.rotary_dim;
+    io.seq_len = 0;
+    io.d_seq_len = s->state + 1;
+    io.max_seq_len = s->desc.cache_rows;
+    return cfpp_neox_layer_decode(&d, &s->layers[l], &io, s->desc.mode, s->ws, s->ws_bytes, st);
+}
+
 int stack_enqueue_step(cfpp_neox_stack* s, hipStream_t st) {
     const cfpp_neox_dims& d = s->desc.dims;
     const int H = d.hidden;
@@ -743,18 +759,7 @@ int stack_enqueue_step(cfpp_neox_stack* s, hipStream_t st) {
     int rc = launch_check();
     if (rc) return rc;
     for (int l = 0; l < s->desc.n_layers; ++l) {
-        cfpp_neox_io io{};
-        io.input = s->hidden[l & 1];
-        io.output = s->hidden[(l + 1) & 1];
-        io.k_new = s->k_new; io.v_new = s->v_new;
-        io.k_cache = s->kc[l]; io.v_cache = s->vc[l];
-        io.cache_rows = s->desc.cache_rows;
-        io.cos = s->desc.rope_cos; io.sin = s->desc.rope_sin;
-        io.rope_stride = d.rotary_dim;
-        io.seq_len = 0;
-        io.d_seq_len = s->state + 1;
-        io.max_seq_len = s->desc.cache_rows;
-        rc = cfpp_neox_layer_decode(&d, &s->layers[l], &io, s->desc.mode, s->ws, s->ws_bytes, st);
+        rc = stack_enqueue_layer(s, l, st);
         if (rc) return rc;
     }
     rc = launch_lm_head(H, s->desc.vocab, d.eps, s->hidden[s->desc.n_layers & 1], s->desc.final_ln_w, s->desc.final_ln_b,
@@ -848,6 +853,54 @@ int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream) {
     for (int i = 0; i < n_steps; ++i) CFPP_HIP(hipGraphLaunch(s->exec, st));
     if (!stream) CFPP_HIP(hipStreamSynchronize(st));
     return CFPP_OK;
+}
+
+int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, float* lm_head_ms, float* total_ms) {
+    if (!s) return CFPP_ERR_NULL;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const int L = s->desc.n_layers;
+    std::vector<hipEvent_t> ev(L + 3);
+    for (auto& e : ev) CFPP_HIP(hipEventCreate(&e));
+    int rc = CFPP_OK;
+    {
+        const cfpp_neox_dims& d = s->desc.dims;
+        const int H = d.hidden;
+        CFPP_HIP(hipEventRecord(ev[L + 2], st));     // start of the step
+        hipLaunchKernelGGL(k_embed, dim3((H / 8 + 255) / 256), dim3(256), 0, st,
+                           reinterpret_cast<const half_t*>(s->desc.embed), s->state, H, s->desc.vocab, s->hidden[0]);
+        rc = launch_check();
+        for (int l = 0; l < L && !rc; ++l) {
+            CFPP_HIP(hipEventRecord(ev[l], st));
+            rc = stack_enqueue_layer(s, l, st);
+        }
+        if (!rc) {
+            CFPP_HIP(hipEventRecord(ev[L], st));
+            rc = launch_lm_head(H, s->desc.vocab, d.eps, s->hidden[L & 1], s->desc.final_ln_w, s->desc.final_ln_b,
+                                s->desc.lm_head, s->logits, s->best_val, s->best_idx, s->grid, st);
+            CFPP_HIP(hipEventRecord(ev[L + 1], st));
+            hipLaunchKernelGGL(k_pick_and_advance, dim3(1), dim3(256), 0, st, s->best_val, s->best_idx, s->grid, s->state,
+                               s->history, s->hist_cap);
+        }
+    }
+    hipEvent_t end;
+    CFPP_HIP(hipEventCreate(&end));
+    CFPP_HIP(hipEventRecord(end, st));
+    CFPP_HIP(hipEventSynchronize(end));
+    if (!rc) {
+        for (int l = 0; l < L; ++l) {
+            float ms = 0.f;
+            CFPP_HIP(hipEventElapsedTime(&ms, ev[l], ev[l + 1]));
+            if (layer_ms) layer_ms[l] = ms;
+        }
+        float ms = 0.f;
+        CFPP_HIP(hipEventElapsedTime(&ms, ev[L], ev[L + 1]));
+        if (lm_head_ms) *lm_head_ms = ms;
+        CFPP_HIP(hipEventElapsedTime(&ms, ev[L + 2], end));
+        if (total_ms) *total_ms = ms;
+    }
+    for (auto& e : ev) (void)hipEventDestroy(e);
+    (void)hipEventDestroy(end);
+    return rc;
 }
 
 int cfpp_stack_buffers(cfpp_neox_stack* s, float** logits, void** hidden, int32_t** state, int32_t** history,

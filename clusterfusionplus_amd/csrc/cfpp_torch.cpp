@@ -289,6 +289,7 @@ struct PyStack {
     std::vector<Tensor> keep;
     cfpp_neox_dims dims{};
     int64_t vocab = 0;
+    int64_t n_layers = 0;
     torch::Device device{torch::kCPU};
     ~PyStack() { if (s) cfpp_stack_destroy(s); }
 };
@@ -339,6 +340,7 @@ std::shared_ptr<PyStack> stack_create(int64_t hidden, int64_t heads, int64_t hea
     c10::hip::HIPGuardMasqueradingAsCUDA guard(embed.device());
     check_rc(cfpp_stack_create(&desc, &ps->s), "stack_create");
     ps->vocab = V;
+    ps->n_layers = L;
     ps->device = embed.device();
     return ps;
 }
@@ -448,6 +450,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         .def("graph_steps", [](PyStack& s, int64_t n) {
             c10::hip::HIPGuardMasqueradingAsCUDA guard(s.device);
             check_rc(cfpp_stack_graph_steps(s.s, (int32_t)n, cur_stream()), "graph_steps");
+        })
+        .def("profile_step", [](PyStack& s) {
+            // (per-layer ms list, lm head ms, whole-step ms) of one eager step timed with HIP events
+            c10::hip::HIPGuardMasqueradingAsCUDA guard(s.device);
+            std::vector<float> layer_ms(s.n_layers, 0.f);
+            float lm = 0.f, total = 0.f;
+            check_rc(cfpp_stack_profile_step(s.s, cur_stream(), layer_ms.data(), &lm, &total), "profile_step");
+            return std::make_tuple(layer_ms, lm, total);
         })
         .def("logits", [](PyStack& s) {
             float* p = nullptr;

@@ -71,6 +71,10 @@ class NeoxDecoder:
         """`n` decode steps, each one replay of the captured hipGraph."""
         self._stack.graph_steps(int(n))
 
+    def profile_step(self):
+        """One eager step with HIP events around every layer launch: (layer_ms list, lm_head_ms, step_ms)."""
+        return self._stack.profile_step()
+
     @property
     def logits(self) -> torch.Tensor:
         return self._stack.logits()

@@ -181,6 +181,10 @@ int cfpp_stack_set_state(cfpp_neox_stack* s, int32_t token, int32_t seq_len, voi
 int cfpp_stack_step(cfpp_neox_stack* s, void* stream);
 /* Captures one step into a hipGraph (first call) and replays it `n_steps` times on `stream`. */
 int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream);
+/* One eager decode step with a HIP event before and after every layer launch and the LM head, on
+ * `stream`; synchronises.  layer_ms[n_layers], *lm_head_ms and *total_ms (whole step) receive elapsed
+ * milliseconds.  For measurement; advances the state like cfpp_stack_step. */
+int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, float* lm_head_ms, float* total_ms);
 /* Device pointers for inspection: logits fp32 [vocab], hidden fp16 [H] after the last layer,
  * state int32[3] = {token, seq_len, steps done}, token history int32 [history_capacity]. */
 int cfpp_stack_buffers(cfpp_neox_stack* s, float** logits, void** hidden, int32_t** state,
