@@ -6,8 +6,9 @@
 //
 //   stage A  LayerNorm statistics in registers of every wave; one wave streams whole weight rows of
 //            W_qkv (then W_up) with 16-byte non-temporal lane loads, 512 contiguous halfs per
-//            wave-load, fp32 accumulation through v_dot2_f32_f16, a DPP row reduction, and a scalar
-//            epilogue (bias -> raw q/k/v in fp32, or bias -> tanh-GELU -> fp16 intermediate).
+//            wave-load, fp32 accumulation through v_dot2_f32_f16 and a DPP row reduction; the dot
+//            products are parked in LDS and finished after the loop, one row per lane
+//            (bias -> raw q/k/v in fp32, or bias -> tanh-GELU -> fp16 intermediate).
 //   stage B  split-KV single-query attention: one wave per (head, KV split); 16 lanes per cache
 //            row, exp2-domain online softmax in fp32, fp32 partials in scratch, and the last wave
 //            to finish a head merges that head's partials in split order.  RoPE is applied when
@@ -70,15 +71,21 @@ struct LayerParams {
     float* part_acc;    // [heads][kMaxSplit][D]
     int* head_cnt;      // [heads] arrival counters, self-resetting
     int* bar;           // device-wide counters, see BarSlot
+    int* grp;           // [events][kEventGroups] group counters, one 64-byte line each
     int* mbox;          // [kMaxGrid][kMailboxInts] event flags, one line per workgroup
     // stage-C selection (split API halves)
     const half_t* c_base0;   // residual terms added to the output (nullable)
     const half_t* c_base1;
     int c_use_o, c_use_down;
+    int dbg;            // TEMP experiment flags
     long long* trace;   // debugging: per-workgroup phase timestamps of the fused kernel (null = off)
 };
 
-constexpr int kTraceSlots = 8;
+constexpr int kTraceSlots = 16;
+__device__ __forceinline__ void trace_value(const LayerParams& p, int slot, long long v) {
+    if (p.trace != nullptr && (threadIdx.x & 63) == 0)
+        p.trace[((size_t)blockIdx.x * kMaxWaves + (threadIdx.x >> 6)) * kTraceSlots + slot] = v;
+}
 __device__ __forceinline__ void trace_mark(const LayerParams& p, int slot) {
     if (p.trace != nullptr && (threadIdx.x & 63) == 0)
         p.trace[((size_t)blockIdx.x * kMaxWaves + (threadIdx.x >> 6)) * kTraceSlots + slot] = wall_clock64();
@@ -191,10 +198,10 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // ------------------------------------------------------------------------------------------------
 // device-wide synchronisation (bounded spins; a timeout raises a status flag and falls through)
 // ------------------------------------------------------------------------------------------------
-// Device-wide events.  Arrivals are counted in one counter per event; the wave whose arrival completes
-// the count writes a flag into one mailbox line per workgroup, and waiters poll only their own
-// workgroup's line.  (Letting every waiting wave poll the shared counter floods a single memory channel
-// with coherent loads and slows the streaming loads of the whole chip.)
+// Device-wide events.  The wave whose arrival completes an event writes a flag into one mailbox line
+// per workgroup, and waiters poll only their own workgroup's line.  (Letting every waiting wave poll a
+// shared counter floods a single memory channel with coherent loads and slows the streaming loads of the
+// whole chip.)
 constexpr int kMailboxInts = 16;       // one 64-byte line per workgroup
 constexpr int kMaxGrid = 1024;         // workgroups a fused launch may have
 
@@ -207,9 +214,44 @@ __device__ __forceinline__ int counter_peek(const int* ctr) {
 __device__ __forceinline__ void raise_status(int* status, int flag) {
     __hip_atomic_fetch_or(status, flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// Called by a whole wave after its stores: drains them, counts the arrival, and if it is the last of
-// `target` arrivals raises mailbox slot `slot` of all `nwg` workgroups.
-__device__ __forceinline__ void event_arrive(int* ctr, int target, int* mbox, int slot, int nwg) {
+// Arrivals are counted hierarchically, because a thousand waves adding to one address serialise at the
+// memory side (tens of nanoseconds each) and every one of them waits for its return value: first in LDS
+// among the waves of a workgroup (when `lds_ctr` is given), then in one of kEventGroups group counters
+// (workgroup index modulo kEventGroups, each on its own 64-byte line), then in the event's top counter.
+// Only the last arrival of each level goes on to the next one.
+constexpr int kEventGroups = 16;
+__device__ __forceinline__ int* group_counter(int* grp, int event, int g) {
+    return grp + (event * kEventGroups + g) * kMailboxInts;
+}
+// Called by a whole wave after its stores: drains them and counts the arrival; `per_wg` waves of every
+// workgroup arrive (1 if lds_ctr is null).  The wave that completes the event raises mailbox slot
+// `event` of all `nwg` workgroups.  Returns true in that wave.
+__device__ __forceinline__ bool event_arrive(int* bar, int* grp, int* mbox, int event, int nwg, int* lds_ctr, int per_wg) {
+    const int lane = threadIdx.x & 63;
+    drain_memory_ops();
+    int go = 1;
+    if (lds_ctr != nullptr) {
+        if (lane == 0) go = (__hip_atomic_fetch_add(lds_ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == per_wg - 1);
+        go = __builtin_amdgcn_readfirstlane(go);
+    }
+    if (!go) return false;
+    const int g = blockIdx.x % kEventGroups;
+    const int gsize = (nwg - g + kEventGroups - 1) / kEventGroups;
+    if (lane == 0) go = (__hip_atomic_fetch_add(group_counter(grp, event, g), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gsize - 1);
+    go = __builtin_amdgcn_readfirstlane(go);
+    if (!go) return false;
+    const int ngroups = nwg < kEventGroups ? nwg : kEventGroups;
+    if (lane == 0) go = (__hip_atomic_fetch_add(bar + event, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngroups - 1);
+    go = __builtin_amdgcn_readfirstlane(go);
+    if (!go) return false;
+    if (mbox != nullptr) {
+        for (int w = lane; w < nwg; w += kWave)
+            __hip_atomic_store(mbox + w * kMailboxInts + event, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return true;
+}
+// A flat count for events with few arrivals (one per attention head).
+__device__ __forceinline__ void event_arrive_flat(int* ctr, int target, int* mbox, int slot, int nwg) {
     const int lane = threadIdx.x & 63;
     drain_memory_ops();
     int last = 0;
@@ -357,19 +399,18 @@ __device__ __forceinline__ void ln_affine(const half_t* __restrict__ x, int H, L
     __builtin_amdgcn_sched_barrier(0);
 }
 
-// RPI weight rows of K = up to NCH*512 halfs held in registers, plus the raw bias of each row.
+// RPI weight rows of K = up to NCH*512 halfs held in registers.
 template <int NCH, int RPI>
 struct RowTile {
     u32x4 w[RPI][NCH];
-    half_t bias[RPI];
 };
 
 // Issue the loads of rows r, r+stride, ... (RPI of them; rows >= nrows repeat row r).  EXACT: K ==
-// NCH*512, every lane load is in range and addresses use immediate offsets; otherwise out-of-range
-// lane loads are redirected to column 0 (their activation registers are zero, so they add nothing).
+// NCH*512, every lane load is in range; otherwise out-of-range lane loads are redirected to column 0
+// (their activation registers are zero, so they add nothing).
 template <int NCH, int RPI, bool EXACT>
-__device__ __forceinline__ void load_row_tile(RowTile<NCH, RPI>& t, const half_t* __restrict__ W, int K,
-                                              const half_t* __restrict__ bias, int r, int stride, int nrows, int lane) {
+__device__ __forceinline__ void load_row_tile(RowTile<NCH, RPI>& t, const half_t* __restrict__ W, int K, int r, int stride,
+                                              int nrows, int lane) {
     const int colb = lane * 8;
 #pragma unroll
     for (int j = 0; j < RPI; ++j) {
@@ -378,64 +419,91 @@ __device__ __forceinline__ void load_row_tile(RowTile<NCH, RPI>& t, const half_t
         const half_t* rp = W + (size_t)rr * (size_t)K;
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
-            const int c = i * kChunk + colb;
-            t.w[j][i] = ld_stream16(rp + ((EXACT || c < K) ? c : 0));
+            if (EXACT) {
+                // scalar base per group of four chunks + one lane offset + immediate: the 13-bit immediate
+                // of a global load reaches 4 KB, and per-chunk lane offsets would cost registers
+                const half_t* gp = rp + (i / 4) * (4 * kChunk);
+                t.w[j][i] = ld_stream16(gp + colb + (i % 4) * kChunk);
+            } else {
+                const int c = i * kChunk + colb;
+                t.w[j][i] = ld_stream16(rp + (c < K ? c : 0));
+            }
         }
-        t.bias[j] = bias ? bias[rr] : (half_t)0.f;
     }
 }
-// epi(row, dot + bias) is called by every lane with wave-uniform arguments
-template <int NCH, int RPI, class Epi>
-__device__ __forceinline__ void finish_row_tile(const RowTile<NCH, RPI>& t, const half2_t (&x)[NCH][4], int r, int stride,
-                                                int nrows, Epi&& epi) {
+
+// Dot products of a wave's rows are parked in LDS (one float per row, written by lane 0) and written to
+// global memory after the streaming loop, one row per lane: a global store inside the loop would share
+// the vmcnt counter with the weight loads, and with loads and stores both pending the compiler has to
+// wait for everything, which empties the load pipeline once per tile.
+constexpr int kParkRows = 64;
+struct RowPark {
+    float* slot;    // this wave's kParkRows floats in LDS
+    int n;          // rows parked so far
+};
+
+template <int NCH, int RPI>
+__device__ __forceinline__ void finish_row_tile(const RowTile<NCH, RPI>& t, const half2_t (&x)[NCH][4], int valid, int lane,
+                                                RowPark& park) {
 #pragma unroll
     for (int j = 0; j < RPI; ++j) {
         float acc = 0.f;
 #pragma unroll
         for (int i = 0; i < NCH; ++i) acc = dot8(t.w[j][i], x[i], acc);
         acc = wave_sum(acc);
-        const int rr = r + j * stride;
-        if (rr < nrows) epi(rr, acc + (float)t.bias[j]);
+        if (j < valid) {
+            if (lane == 0) park.slot[park.n] = acc;
+            park.n += 1;
+        }
     }
 }
 
-// Rows first, first+stride, ... < nrows, RPI rows per tile, two tiles in flight: the loads of the next
-// tile are issued before the current one is reduced, so a wave keeps up to 2*RPI*NCH KB outstanding.
-// `pre` already holds the loads of the first tile (issued by the caller before something slow: the
-// LayerNorm prologue or a barrier).
-template <int NCH, int RPI, bool EXACT, class Epi>
-__device__ __forceinline__ void gemv_rows(const half_t* __restrict__ W, int K, const half_t* __restrict__ bias, int first,
-                                          int stride, int nrows, const half2_t (&x)[NCH][4], int lane,
-                                          RowTile<NCH, RPI>& pre, Epi&& epi) {
-    const int step = stride * RPI;
-    int r = first;
-    if (r >= nrows) return;
-    RowTile<NCH, RPI> other;
-    for (;;) {
-        const int r2 = r + step;
-        if (r2 < nrows) load_row_tile<NCH, RPI, EXACT>(other, W, K, bias, r2, stride, nrows, lane);
-        finish_row_tile<NCH, RPI>(pre, x, r, stride, nrows, epi);
-        __builtin_amdgcn_sched_barrier(0);   // a third tile's loads must not be scheduled above this point
-        if (r2 >= nrows) break;
-        r = r2 + step;
-        if (r < nrows) load_row_tile<NCH, RPI, EXACT>(pre, W, K, bias, r, stride, nrows, lane);
-        finish_row_tile<NCH, RPI>(other, x, r2, stride, nrows, epi);
-        __builtin_amdgcn_sched_barrier(0);
-        if (r >= nrows) break;
+// Tiles t = 0 .. ntiles-1 of one wave: tile t covers rows row_of(t) + j*stride_in_tile, j < RPI (rows >=
+// nrows do not exist).  Two tiles are in flight: the loads of the next tile are issued before the current
+// one is reduced.  `pre` already holds the loads of tile 0 (issued by the caller before something slow:
+// the LayerNorm prologue or a barrier).  The loop body is free of branches: the loads of a tile past the
+// end re-read the last tile instead of being skipped, because a conditional load makes the compiler's
+// wait-count bookkeeping assume the shorter path and drain the pipeline at every tile.
+// The tiles are processed in segments of kParkRows rows; `flush(park, first_index)` runs after each
+// segment, outside the streaming loop (no global store may sit inside it, see RowPark); parked value k
+// (counting from first_index) belongs to the k-th row this wave finished.
+template <int NCH, int RPI, bool EXACT, class RowOf, class Flush>
+__device__ __forceinline__ void gemv_tiles(const half_t* __restrict__ W, int K, int nrows, int stride_in_tile, int ntiles,
+                                           RowOf&& row_of, const half2_t (&x)[NCH][4], int lane, RowTile<NCH, RPI>& pre,
+                                           RowPark& park, Flush&& flush) {
+    constexpr int kSegTiles = (kParkRows / RPI) & ~1;   // even, so a segment is a whole number of loop trips
+    static_assert(kSegTiles >= 2, "tile larger than the park");
+    auto valid_rows = [&](int t) {
+        int v = 0;
+        if (t < ntiles) {
+            const int r = row_of(t);
+#pragma unroll
+            for (int j = 0; j < RPI; ++j) v += (r + j * stride_in_tile < nrows) ? 1 : 0;
+        }
+        return v;
+    };
+    auto tile_row = [&](int t) { return row_of(t < ntiles ? t : ntiles - 1); };
+    int done = 0;
+    for (int seg = 0; seg < ntiles; seg += kSegTiles) {
+        const int seg_end = seg + kSegTiles < ntiles ? seg + kSegTiles : ntiles;
+        if (seg != 0) load_row_tile<NCH, RPI, EXACT>(pre, W, K, tile_row(seg), stride_in_tile, nrows, lane);
+        RowTile<NCH, RPI> other;
+        for (int t = seg; t < seg_end; t += 2) {
+            load_row_tile<NCH, RPI, EXACT>(other, W, K, tile_row(t + 1), stride_in_tile, nrows, lane);
+            finish_row_tile<NCH, RPI>(pre, x, valid_rows(t), lane, park);
+            __builtin_amdgcn_sched_barrier(0);   // a third tile's loads must not be scheduled above this point
+            load_row_tile<NCH, RPI, EXACT>(pre, W, K, tile_row(t + 2), stride_in_tile, nrows, lane);
+            finish_row_tile<NCH, RPI>(other, x, t + 1 < seg_end ? valid_rows(t + 1) : 0, lane, park);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        flush(park, done);
+        done += park.n;
+        park.n = 0;
     }
 }
 
 template <int NCH>
 struct StageARpi { static constexpr int value = (16 / NCH) > 0 ? (16 / NCH) : 1; };
-
-__device__ __forceinline__ auto qkv_epilogue(const LayerParams& p, int lane) {
-    float* __restrict__ dst = p.qkv_raw;
-    return [dst, lane](int r, float v) { if (lane == 0) st_agent(dst + r, v); };
-}
-__device__ __forceinline__ auto up_epilogue(const LayerParams& p, int lane) {
-    half_t* __restrict__ dst = p.inter;
-    return [dst, lane](int r, float v) { if (lane == 0) st_agent(dst + r, (half_t)gelu_tanh(v)); };
-}
 
 // ------------------------------------------------------------------------------------------------
 // stage B: split-KV single-query attention, one wave per (head, split) item
@@ -632,7 +700,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
             st_agent(reinterpret_cast<uint32_t*>(p.attn_vec + (size_t)head * D + t2), as_u32(o));
         }
         if (lane == 0) __hip_atomic_store(p.head_cnt + head, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (nwg_to_signal > 0) event_arrive(p.bar + kBarHeads, p.heads, p.mbox, kBarHeads, nwg_to_signal);
+        if (nwg_to_signal > 0) event_arrive_flat(p.bar + kBarHeads, p.heads, p.mbox, kBarHeads, nwg_to_signal);
     }
 }
 
@@ -696,10 +764,11 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
     for (int b0 = r0; b0 < r1; b0 += kRowBatch) {
         const int b1 = (b0 + kRowBatch < r1) ? b0 + kRowBatch : r1;
         if (wave < kStreamers) {
+            // rows past the batch re-read its last row (no conditional loads, see gemv_tiles)
             auto load_rows = [&](u32x4 (&w)[RPI][CP], int r) {
 #pragma unroll
                 for (int j = 0; j < RPI; ++j) {
-                    const int rr = (r + j < b1) ? r + j : r;
+                    const int rr = (r + j < b1) ? r + j : b1 - 1;
 #pragma unroll
                     for (int i = 0; i < CP; ++i) w[j][i] = ld_stream16(wp[i] + (size_t)rr * wstride[i]);
                 }
@@ -725,18 +794,13 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
                     xs[i][0] = as_h2(xv.x); xs[i][1] = as_h2(xv.y); xs[i][2] = as_h2(xv.z); xs[i][3] = as_h2(xv.w);
                 }
             }
-            int r = b0;
-            for (;;) {
-                const int r2 = r + RPI;
-                if (r2 < b1) load_rows(wb, r2);
+            for (int r = b0; r < b1; r += 2 * RPI) {   // two tiles in flight, branch-free body
+                load_rows(wb, r + RPI);
                 finish_rows(wa, r);
                 __builtin_amdgcn_sched_barrier(0);   // a third tile's loads must not be scheduled above this point
-                if (r2 >= b1) break;
-                r = r2 + RPI;
-                if (r < b1) load_rows(wa, r);
-                finish_rows(wb, r2);
+                load_rows(wa, r + 2 * RPI);
+                finish_rows(wb, r + RPI);
                 __builtin_amdgcn_sched_barrier(0);
-                if (r >= b1) break;
             }
         }
         first = false;

@@ -23,27 +23,49 @@ namespace {
 
 // EX (hidden == NCH*512) is a template parameter of every kernel, chosen by the host: a run-time branch
 // between the two variants makes the compiler keep two copies of the in-flight tiles.
-// MLP-up rows of one wave: batches first, first+stride, ... of kUpRpi adjacent rows, two batches in flight
+
+// QKV rows of one streaming wave: rows first, first+stride, ...; result = dot + bias as raw fp32.
 template <int NCH, bool EX>
-__device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], int first, int stride, int lane) {
+__device__ __forceinline__ void qkv_rows(const LayerParams& p, const half2_t (&x1)[NCH][4], int first, int stride, int lane,
+                                         RowTile<NCH, StageARpi<NCH>::value>& pre, RowPark& park) {
+    constexpr int RPI = StageARpi<NCH>::value;
+    const int nq = 3 * p.H;
+    const int mine = first < nq ? (nq - first + stride - 1) / stride : 0;      // rows of this wave
+    gemv_tiles<NCH, RPI, EX>(
+        p.w_qkv, p.H, nq, stride, (mine + RPI - 1) / RPI, [=](int t) { return first + t * RPI * stride; }, x1, lane, pre, park,
+        [&](const RowPark& pk, int k0) {
+            if (lane < pk.n) {
+                const int row = first + (k0 + lane) * stride;
+                st_agent(p.qkv_raw + row, pk.slot[lane] + (float)p.b_qkv[row]);
+            }
+        });
+}
+template <int NCH, bool EX>
+__device__ __forceinline__ void qkv_prefetch(const LayerParams& p, int first, int stride, int lane,
+                                             RowTile<NCH, StageARpi<NCH>::value>& pre) {
+    const int nq = 3 * p.H;
+    if (first < nq) load_row_tile<NCH, StageARpi<NCH>::value, EX>(pre, p.w_qkv, p.H, first, stride, nq, lane);
+}
+
+// MLP-up rows of one streaming wave: batches first, first+stride, ... of kUpRpi adjacent rows;
+// result = gelu(dot + bias) as fp16.
+template <int NCH, bool EX>
+__device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], int first, int stride, int lane,
+                                        RowPark& park) {
     const int nbatch = (p.F + kUpRpi - 1) / kUpRpi;
-    int j = first;
-    if (j >= nbatch) return;
-    auto epi = up_epilogue(p, lane);
-    RowTile<NCH, kUpRpi> ta, tb;
-    load_row_tile<NCH, kUpRpi, EX>(ta, p.w_up, p.H, p.b_up, j * kUpRpi, 1, p.F, lane);
-    for (;;) {
-        const int j2 = j + stride;
-        if (j2 < nbatch) load_row_tile<NCH, kUpRpi, EX>(tb, p.w_up, p.H, p.b_up, j2 * kUpRpi, 1, p.F, lane);
-        finish_row_tile<NCH, kUpRpi>(ta, x2, j * kUpRpi, 1, p.F, epi);
-        __builtin_amdgcn_sched_barrier(0);
-        if (j2 >= nbatch) break;
-        j = j2 + stride;
-        if (j < nbatch) load_row_tile<NCH, kUpRpi, EX>(ta, p.w_up, p.H, p.b_up, j * kUpRpi, 1, p.F, lane);
-        finish_row_tile<NCH, kUpRpi>(tb, x2, j2 * kUpRpi, 1, p.F, epi);
-        __builtin_amdgcn_sched_barrier(0);
-        if (j >= nbatch) break;
-    }
+    const int mine = first < nbatch ? (nbatch - first + stride - 1) / stride : 0;   // batches of this wave
+    if (mine == 0) return;
+    RowTile<NCH, kUpRpi> pre;
+    load_row_tile<NCH, kUpRpi, EX>(pre, p.w_up, p.H, first * kUpRpi, 1, p.F, lane);
+    gemv_tiles<NCH, kUpRpi, EX>(
+        p.w_up, p.H, p.F, 1, mine, [=](int t) { return (first + t * stride) * kUpRpi; }, x2, lane, pre, park,
+        [&](const RowPark& pk, int k0) {
+            if (lane < pk.n) {
+                const int k = k0 + lane;
+                const int row = (first + (k / kUpRpi) * stride) * kUpRpi + (k % kUpRpi);
+                st_agent(p.inter + row, (half_t)gelu_tanh(pk.slot[lane] + (float)p.b_up[row]));
+            }
+        });
 }
 
 // ---- split mode: one launch per stage ----------------------------------------------------------
@@ -51,17 +73,17 @@ __device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2
 // memory pipeline than the first while both stream, so extra streaming waves only add imbalance.
 template <int NCH, bool EX>
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_a(LayerParams p) {
+    __shared__ float park_mem[kStreamers][kParkRows];
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int gw = blockIdx.x * kStreamers + wave, nw = gridDim.x * kStreamers;
-    constexpr int RPIA = StageARpi<NCH>::value;
-    const int nq = 3 * p.H;
-    RowTile<NCH, RPIA> t0;
-    if (gw < nq) load_row_tile<NCH, RPIA, EX>(t0, p.w_qkv, p.H, p.b_qkv, gw, nw, nq, lane);
+    RowPark park{park_mem[wave], 0};
+    RowTile<NCH, StageARpi<NCH>::value> t0;
+    qkv_prefetch<NCH, EX>(p, gw, nw, lane, t0);
     half2_t xr[NCH][4];
     const LnStats st = ln_first<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, lane, xr);
-    gemv_rows<NCH, RPIA, EX>(p.w_qkv, p.H, p.b_qkv, gw, nw, nq, xr, lane, t0, qkv_epilogue(p, lane));
+    qkv_rows<NCH, EX>(p, xr, gw, nw, lane, t0, park);
     ln_affine<NCH>(p.x, p.H, st, p.ln2_w, p.ln2_b, lane, xr);
-    up_rows<NCH, EX>(p, xr, gw, nw, lane);
+    up_rows<NCH, EX>(p, xr, gw, nw, lane, park);
 }
 
 // one (head, split) item per wave
@@ -91,7 +113,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
 //                   trips; it runs beside the MLP-up streaming instead of in front of it.
 // The last workgroup to leave zeroes the counters for the next launch.  All workgroups must be
 // co-resident (the host launches one per compute unit); every wait is bounded.
-struct FusedShared { int attn_next; };
+struct FusedShared { int attn_next; int arrived[2]; };
 
 __device__ __forceinline__ int lds_take(int* p) { return __hip_atomic_fetch_add(p, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 
@@ -99,18 +121,22 @@ template <int NCH, int CPC, bool EX>
 __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     __shared__ FusedShared q;
     __shared__ StageCShared shc;
+    __shared__ float park_mem[kStreamers][kParkRows];
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int G = gridDim.x, b = blockIdx.x;
     const int nsw = G * kStreamers;                 // streaming waves in the grid
     int* status = p.bar + kBarStatus;
-    if (threadIdx.x == 0) q.attn_next = 0;
+    if (threadIdx.x == 0) { q.attn_next = 0; q.arrived[0] = 0; q.arrived[1] = 0; }
     __syncthreads();
     trace_mark(p, 0);
+    trace_value(p, 8, __builtin_amdgcn_s_getreg((3 << 11) | 20));   // XCC_ID: which XCD this workgroup runs on
+    trace_value(p, 11, __builtin_amdgcn_s_getreg((31 << 11) | 4));  // HW_ID: wave slot, SIMD, CU, SE
 
     const int S = load_seq_len(p);
     const int nsplit = effective_split(p, S);
     const int nitems = p.heads * nsplit;
-    const int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
+    int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
+    if (p.dbg & 1) attn_count = 0;
     auto take_attention_items = [&] {
         for (;;) {
             int t = 0;
@@ -126,45 +152,50 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
 
     if (wave < kStreamers) {
         const int sgw = b * kStreamers + wave;
-        constexpr int RPIA = StageARpi<NCH>::value;
-        const int nq = 3 * p.H;
+        RowPark park{park_mem[wave], 0};
         half2_t xr[NCH][4];   // ln1(x) for the QKV rows, then ln2(x) for the MLP-up rows
-        RowTile<NCH, RPIA> t0;
-        if (sgw < nq) load_row_tile<NCH, RPIA, EX>(t0, p.w_qkv, p.H, p.b_qkv, sgw, nsw, nq, lane);
+        RowTile<NCH, StageARpi<NCH>::value> t0;
+        qkv_prefetch<NCH, EX>(p, sgw, nsw, lane, t0);
         const LnStats st = ln_first<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, lane, xr);
         trace_mark(p, 1);
-        gemv_rows<NCH, RPIA, EX>(p.w_qkv, p.H, p.b_qkv, sgw, nsw, nq, xr, lane, t0, qkv_epilogue(p, lane));
-        event_arrive(p.bar + kBarQkv, nsw, p.mbox, kBarQkv, G);
+        qkv_rows<NCH, EX>(p, xr, sgw, nsw, lane, t0, park);
+        event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], kStreamers);
         trace_mark(p, 2);
         ln_affine<NCH>(p.x, p.H, st, p.ln2_w, p.ln2_b, lane, xr);
-        up_rows<NCH, EX>(p, xr, sgw, nsw, lane);
-        event_arrive(p.bar + kBarUp, nsw, p.mbox, kBarUp, G);
+        up_rows<NCH, EX>(p, xr, sgw, nsw, lane, park);
+        event_arrive(p.bar, p.grp, p.mbox, kBarUp, G, &q.arrived[1], kStreamers);
         trace_mark(p, 5);
         event_wait(p.mbox, kBarQkv, status);
         take_attention_items();
-    } else {
+    } else if (!(p.dbg & 2)) {
         event_wait(p.mbox, kBarQkv, status);
         __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
         take_attention_items();
         __builtin_amdgcn_s_setprio(0);
     }
+    trace_mark(p, 9);
     {
         const StageC c = make_stage_c(p);
         stage_c_rows<CPC>(c, b, G, shc, [&] {
             event_wait(p.mbox, kBarUp, status);
             trace_mark(p, 6);
-            event_wait(p.mbox, kBarHeads, status);
+            if (!(p.dbg & 1)) event_wait(p.mbox, kBarHeads, status);
             trace_mark(p, 7);
         });
     }
+    trace_mark(p, 10);
     // the last workgroup to leave re-arms the counters and mailboxes for the next launch
     __shared__ int last_out;
-    if (threadIdx.x == 0)
-        last_out = (__hip_atomic_fetch_add(p.bar + kBarExit, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == G - 1);
+    if (wave == 0) {
+        const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1);
+        if (lane == 0) last_out = last;
+    }
     __syncthreads();
     if (last_out) {
         for (int i = threadIdx.x; i < G * kMailboxInts; i += blockDim.x)
             __hip_atomic_store(p.mbox + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int i = threadIdx.x; i < (kBarExit + 1) * kEventGroups * kMailboxInts; i += blockDim.x)
+            __hip_atomic_store(p.grp + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (threadIdx.x <= kBarExit) __hip_atomic_store(p.bar + threadIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
@@ -191,16 +222,32 @@ __global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __res
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int gw = blockIdx.x * NWV + wave, nw = gridDim.x * NWV;
     constexpr int RPIA = StageARpi<NCH>::value;
+    __shared__ float park_mem[NWV][kParkRows];
+    RowPark park{park_mem[wave], 0};
     RowTile<NCH, RPIA> t0;
-    if (gw < vocab) load_row_tile<NCH, RPIA, EX>(t0, W, H, nullptr, gw, nw, vocab, lane);
+    if (gw < vocab) load_row_tile<NCH, RPIA, EX>(t0, W, H, gw, nw, vocab, lane);
     half2_t x1[NCH][4];
     ln_first<NCH>(x, H, eps, ln_w, ln_b, lane, x1);
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    gemv_rows<NCH, RPIA, EX>(W, H, nullptr, gw, nw, vocab, x1, lane, t0, [&](int r, float v) {
-        if (lane == 0) logits[r] = v;
-        if (v > bv || (v == bv && r < bi)) { bv = v; bi = r; }
-    });
+    const int mine = gw < vocab ? (vocab - gw + nw - 1) / nw : 0;
+    gemv_tiles<NCH, RPIA, EX>(
+        W, H, vocab, nw, (mine + RPIA - 1) / RPIA, [=](int t) { return gw + t * RPIA * nw; }, x1, lane, t0, park,
+        [&](const RowPark& pk, int k0) {
+            if (lane < pk.n) {
+                const int row = gw + (k0 + lane) * nw;
+                const float v = pk.slot[lane];
+                logits[row] = v;
+                if (v > bv || (v == bv && row < bi)) { bv = v; bi = row; }
+            }
+        });
+    // lanes hold the best of the rows they wrote: reduce over the wave (ties to the lower index)
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const float ov = xor_shfl(bv, m);
+        const int oi = __shfl_xor(bi, m, kWave);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
     if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -281,7 +328,7 @@ constexpr size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 long long* g_trace = nullptr;   // see cfpp_debug_set_trace
 
 struct WorkspaceLayout {
-    size_t qkv_raw, attn_vec, inter, part_ml, part_acc, head_cnt, bar, mbox, total;
+    size_t qkv_raw, attn_vec, inter, part_ml, part_acc, head_cnt, bar, grp, mbox, total;
 };
 
 WorkspaceLayout workspace_layout(const cfpp_neox_dims& d) {
@@ -295,6 +342,7 @@ WorkspaceLayout workspace_layout(const cfpp_neox_dims& d) {
     w.part_acc = take((size_t)d.heads * kMaxSplit * d.head_dim * 4);
     w.head_cnt = take((size_t)d.heads * 4);
     w.bar = take(64);
+    w.grp = take((size_t)(kBarExit + 1) * kEventGroups * kMailboxInts * 4);
     w.mbox = take((size_t)kMaxGrid * kMailboxInts * 4);
     w.total = off;
     return w;
@@ -449,9 +497,11 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     p.part_acc = reinterpret_cast<float*>(ws + L.part_acc);
     p.head_cnt = reinterpret_cast<int*>(ws + L.head_cnt);
     p.bar = reinterpret_cast<int*>(ws + L.bar);
+    p.grp = reinterpret_cast<int*>(ws + L.grp);
     p.mbox = reinterpret_cast<int*>(ws + L.mbox);
     p.c_base0 = p.x; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 1;
     p.trace = g_trace;
+    p.dbg = env_int("CFPP_DBG", 0);
     *out = p;
     return CFPP_OK;
 }

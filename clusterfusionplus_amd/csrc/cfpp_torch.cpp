@@ -399,10 +399,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
 
     m.def("cfpp_version", []() { return std::string(cfpp_version()); });
     m.def("debug_set_trace", [](c10::optional<Tensor> buf) {
-        // int64 device tensor of at least 1024*16*8 elements, or None to switch tracing off
+        // int64 device tensor of at least 1024*16*16 elements, or None to switch tracing off
         if (buf.has_value()) {
-            TORCH_CHECK(buf->is_cuda() && buf->scalar_type() == torch::kInt64 && buf->is_contiguous() && buf->numel() >= 1024 * 16 * 8,
-                        "trace buffer must be a contiguous int64 GPU tensor with >= 131072 elements");
+            TORCH_CHECK(buf->is_cuda() && buf->scalar_type() == torch::kInt64 && buf->is_contiguous() && buf->numel() >= 1024 * 16 * 16,
+                        "trace buffer must be a contiguous int64 GPU tensor with >= 262144 elements");
             cfpp_debug_set_trace(buf->data_ptr());
         } else {
             cfpp_debug_set_trace(nullptr);

@@ -147,7 +147,7 @@ int cfpp_workspace_check(const cfpp_neox_dims* dims, void* workspace, void* stre
 
 /* Debugging aid: when set to a device buffer of cfpp_debug_trace_bytes() bytes, every fused launch
  * stores 100 MHz timestamps of its phase boundaries per workgroup and wave
- * ([workgroup][16 waves][8 slots] int64); NULL switches it off.  No counterpart in the reference. */
+ * ([workgroup][16 waves][16 slots] int64); NULL switches it off.  No counterpart in the reference. */
 int cfpp_debug_set_trace(void* device_buffer);
 
 /* ---- whole-model greedy decode (our counterpart of the reference's Python decode loop,
