@@ -14,10 +14,10 @@
 //            to finish a head merges that head's partials in split order.  RoPE is applied when
 //            q / k are read from the raw fp32 scratch; the (head, split 0) wave appends the rotated
 //            K and V to the cache and returns them.
-//   stage C  out = x + b_o + b_down + W_o attn + W_down h as one GEMV over the concatenated input;
-//            the K dimension is split over the waves of a workgroup (the activation slice lives in
-//            registers), rows are split over workgroups, and a fixed-order LDS reduction finishes
-//            each row: deterministic, no atomics on data.
+//   stage C  out = x + b_o + b_down + W_o attn + W_down h; rows are split over workgroups.  MLP-down
+//            is K-split over the streaming waves of a workgroup (activation slices in registers),
+//            the O projection is row-per-wave; a fixed-order LDS reduction finishes each row:
+//            deterministic, no atomics on data.
 //
 // The same device functions are used by the per-stage kernels (split mode: the kernel boundary is
 // the barrier) and by the persistent fused kernel (device-wide barriers with bounded waits).
@@ -77,7 +77,6 @@ struct LayerParams {
     const half_t* c_base0;   // residual terms added to the output (nullable)
     const half_t* c_base1;
     int c_use_o, c_use_down;
-    int dbg;            // TEMP experiment flags
     long long* trace;   // debugging: per-workgroup phase timestamps of the fused kernel (null = off)
 };
 
@@ -342,15 +341,9 @@ __device__ __forceinline__ void ln_load3(const half_t* __restrict__ x, const hal
 template <int NCH>
 __device__ __forceinline__ LnStats ln_first(const half_t* __restrict__ x, int H, float eps, const half_t* __restrict__ w,
                                             const half_t* __restrict__ b, int lane, half2_t (&dst)[NCH][4]) {
-    // x first; the affine vectors are fetched after the statistics (they are cache resident: every
-    // workgroup reads the same few KB), which keeps fewer registers live beside a prefetched weight tile
-    u32x4 rx[NCH];
-    const u32x4 z = {0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        const int col = i * kChunk + lane * 8;
-        rx[i] = col < H ? ld16(x + col) : z;
-    }
+    // x and the affine vectors are requested together: one memory round trip for the prologue
+    u32x4 rx[NCH], rw[NCH], rb[NCH];
+    ln_load3<NCH>(x, w, b, H, lane, rx, rw, rb);
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
@@ -376,13 +369,6 @@ __device__ __forceinline__ LnStats ln_first(const half_t* __restrict__ x, int H,
     st.rstd = 1.0f / sqrtf(wave_sum(q) / (float)H + eps);
 #pragma unroll
     for (int i = 0; i < NCH; ++i) keep_packed(rx[i]);
-    u32x4 rw[NCH], rb[NCH];
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        const int col = i * kChunk + lane * 8;
-        rw[i] = col < H ? ld16(w + col) : z;
-        rb[i] = col < H ? ld16(b + col) : z;
-    }
     ln_apply<NCH>(rx, rw, rb, H, st, lane, dst);
     // keep later weight loads from being scheduled up into the prologue (they would only add register pressure)
     __builtin_amdgcn_sched_barrier(0);
@@ -539,16 +525,37 @@ __device__ __forceinline__ void rope_load8(const float* __restrict__ v, int d0, 
 }
 
 // The wave's four 16-lane groups take cache rows begin+g, begin+g+4, ...; lane `sub` of a group holds
-// dims 8 sub .. 8 sub + 7 of its row (lanes with 8 sub >= D idle).  T rows per group are in flight.
+// dims 8 sub .. 8 sub + 7 of its row (lanes with 8 sub >= D contribute nothing).  T rows per group are in
+// flight (32 rows per wave).  An item is a chain of dependent memory round trips, so everything that can
+// be requested early is: the first K/V tile goes out before q is fetched.
 // nwg_to_signal > 0 (fused kernel): a completed head counts towards the kBarHeads event of that many workgroups.
 __device__ __forceinline__ void attention_item(const LayerParams& p, int head, int sp, int nsplit, int S, int lane,
                                                int nwg_to_signal) {
     const int grp = lane >> 4, sub = lane & 15;
-    const int D = p.D, H = p.H, d0 = sub * 8;
-    const bool act = d0 < D;
+    const int D = p.D, H = p.H;
+    const bool act = sub * 8 < D;
+    const int d0 = act ? sub * 8 : 0;      // idle lanes read (and ignore) the first dims
     const float* __restrict__ raw = p.qkv_raw + (size_t)head * 3 * D;
     const float* __restrict__ cs = p.cos + (size_t)S * p.rope_stride;   // stride 0: the row is the position
     const float* __restrict__ sn = p.sin + (size_t)S * p.rope_stride;
+
+    const int chunk = (S + nsplit - 1) / nsplit;
+    const int begin = sp * chunk;
+    const int end = (begin + chunk < S) ? begin + chunk : S;
+    const half_t* __restrict__ kc = p.k_cache + (size_t)head * D + d0;
+    const half_t* __restrict__ vc = p.v_cache + (size_t)head * D + d0;
+    constexpr int T = 8;
+    u32x4 kk[T], vv[T];
+    // rows past the end re-read the last row (masked below): no conditional loads
+    auto load_kv = [&](int r) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const int row = (r + t * 4 < end) ? r + t * 4 : end - 1;
+            kk[t] = ld16(kc + (size_t)row * H);
+            vv[t] = ld16(vc + (size_t)row * H);
+        }
+    };
+    if (begin < end) load_kv(begin + grp);
 
     float q[8];
     rope_load8(raw, d0, p.rot, cs, sn, act, q);
@@ -584,26 +591,8 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
         for (int j = 0; j < 8; ++j) acc[j] = vf[j];
     }
 
-    const int chunk = (S + nsplit - 1) / nsplit;
-    const int begin = sp * chunk;
-    const int end = (begin + chunk < S) ? begin + chunk : S;
-    const half_t* __restrict__ kc = p.k_cache + (size_t)head * D + d0;
-    const half_t* __restrict__ vc = p.v_cache + (size_t)head * D + d0;
-    constexpr int T = 8;
-    for (int r = begin + grp; r < end; r += 4 * T) {
-        u32x4 kk[T], vv[T];
-        bool ok[T];
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-            const int row = r + t * 4;
-            ok[t] = row < end;
-            const u32x4 z = {0u, 0u, 0u, 0u};
-            kk[t] = z; vv[t] = z;
-            if (ok[t] && act) {
-                kk[t] = ld16(kc + (size_t)row * H);
-                vv[t] = ld16(vc + (size_t)row * H);
-            }
-        }
+    for (int r = begin + grp; r - grp < end; r += 4 * T) {
+        if (r - grp != begin) load_kv(r);
         float s[T], mt = m;
 #pragma unroll
         for (int t = 0; t < T; ++t) {
@@ -613,7 +602,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
 #pragma unroll
             for (int j = 0; j < 8; ++j) d += q[j] * kf[j];
             d = row16_sum(d);
-            s[t] = ok[t] ? d : kNegBig;
+            s[t] = (r + t * 4 < end) ? d : kNegBig;
             mt = fmaxf(mt, s[t]);
         }
         const float alpha = fast_exp2(m - mt);
@@ -622,7 +611,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
         for (int j = 0; j < 8; ++j) acc[j] *= alpha;
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-            const float pt = ok[t] ? fast_exp2(s[t] - mt) : 0.f;
+            const float pt = (r + t * 4 < end) ? fast_exp2(s[t] - mt) : 0.f;
             float vf[8];
             unpack8(vv[t], vf);
             l += pt;
@@ -663,7 +652,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
     last = first_lane(last);
     if (last) {
         // The last wave of this head merges the splits.  Lane i fetches (m_i, l_i) of split i, so the
-        // scales come from one round trip; the accumulators (two dims per lane) are fetched eight
+        // scales come from one round trip; the accumulators (two dims per lane) are fetched 16
         // splits at a time and added in split order.
         const size_t hb = (size_t)head * kMaxSplit;
         float mi = kNegBig, li = 0.f;
@@ -679,18 +668,19 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
         const int t2 = lane * 2;
         const bool dact = t2 < D;
         float L = 0.f, A0 = 0.f, A1 = 0.f;
-        for (int i0 = 0; i0 < nsplit; i0 += 8) {
-            float a0[8], a1[8];
+        for (int i0 = 0; i0 < nsplit; i0 += 16) {     // 16 splits per memory round trip
+            float a0[16], a1[16];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                a0[u] = 0.f; a1[u] = 0.f;
-                if (dact && i0 + u < nsplit) ld_agent2(p.part_acc + (hb + i0 + u) * D + t2, a0[u], a1[u]);
+            for (int u = 0; u < 16; ++u) {
+                const int i = i0 + u < nsplit ? i0 + u : nsplit - 1;
+                ld_agent2(p.part_acc + (hb + i) * D + (dact ? t2 : 0), a0[u], a1[u]);
             }
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int i = i0 + u < nsplit ? i0 + u : 0;
-                const float sc = i0 + u < nsplit ? rl(sci, i) : 0.f;
-                L += i0 + u < nsplit ? rl(lsi, i) : 0.f;
+            for (int u = 0; u < 16; ++u) {
+                const bool in = i0 + u < nsplit;
+                const int i = in ? i0 + u : 0;
+                const float sc = in ? rl(sci, i) : 0.f;
+                L += in ? rl(lsi, i) : 0.f;
                 A0 += a0[u] * sc;
                 A1 += a1[u] * sc;
             }
@@ -724,76 +714,73 @@ __device__ __forceinline__ StageC make_stage_c(const LayerParams& p) {
 }
 
 constexpr int kStreamers = 4;          // streaming waves per workgroup: one per SIMD of the compute unit
-struct StageCShared { float red[kRowBatch][kStreamers]; };
+struct StageCShared {
+    float red_down[kRowBatch][kStreamers];   // MLP-down partials of the K slices
+    float red_o[kRowBatch];                  // O-projection dot products
+};
 
-// Stage C for the rows of workgroup `wg`: one GEMV over the concatenated input [x1 | x2].  Called by
-// every wave of the workgroup; waves >= kStreamers only take part in the workgroup barriers.
-// K is cut into 512-half chunks over the concatenation; streaming wave ks owns chunks ks, ks+4, ...
-// (at most CP), keeps its slices of x in registers, streams RPI rows per tile with two tiles in flight,
-// and leaves its partial dot product of every row in LDS; the partials are then added in wave order
-// together with the biases and residual terms: deterministic, and identical in both modes.
-// `ready()` runs after the loads of the first tile are in flight and before x is read (x is produced by
-// other workgroups; the fused kernel waits for it there, so the wait overlaps the loads).
-template <int CP, class Ready>
-__device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, StageCShared& sh, Ready&& ready) {
-    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+// Stage C for the rows of workgroup `wg`, as two independent GEMVs whose results meet in LDS:
+//   MLP down   K-split over the kStreamers streaming waves (wave ks owns the 512-half chunks ks, ks+4, ...
+//              of W2 and x2, at most CPD of them, activation slices in registers), RPI rows per tile, two
+//              tiles in flight; each wave leaves its partial dot product of every row in red_down.
+//   O proj     row-per-wave over the `n_o` waves that have o_index >= 0 (row b0 + o_index, + n_o, ...),
+//              the whole attention vector in registers (K1 <= NCH*512), two rows in flight; red_o.
+// In the fused kernel the streaming waves do the MLP-down part and the helper waves the O projection,
+// so the attention output is not needed until the (longer) MLP-down pass is over; in split mode the same
+// four waves do one after the other.  `down_ready()` / `o_ready()` run after the first loads of a pass are
+// in flight and before its activations are read (the fused kernel waits for the producing event there).
+// The partials are added in a fixed order with the biases and residual terms: deterministic, and
+// identical in both modes.  Every wave of the workgroup must call this (workgroup barriers inside).
+template <int NCH, int CPD, class DownReady, class OReady>
+__device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, StageCShared& sh, bool streamer, int ks,
+                                             int o_index, int n_o, DownReady&& down_ready, OReady&& o_ready) {
+    const int lane = threadIdx.x & 63;
     const int r0 = (int)(((long long)wg * c.nrows) / nwg), r1 = (int)(((long long)(wg + 1) * c.nrows) / nwg);
-    constexpr int RPI = (16 / CP) > 0 ? (16 / CP) : 1;
-    const int nch1 = (c.K1 + kChunk - 1) / kChunk, nch2 = (c.K2 + kChunk - 1) / kChunk;
-
-    // per-chunk row-0 pointer and row stride; a chunk that does not exist for this lane reads a valid
-    // dummy location with stride 0 and a zero activation slice
-    const half_t* wp[CP];
-    const half_t* xp[CP];
-    int wstride[CP];
-    const half_t* dummy = c.W1 ? c.W1 : c.W2;
-#pragma unroll
-    for (int i = 0; i < CP; ++i) {
-        const int ch = wave + i * kStreamers;
-        wp[i] = dummy; wstride[i] = 0; xp[i] = nullptr;
-        if (ch < nch1) {
-            const int col = ch * kChunk + lane * 8;
-            if (col < c.K1) { wp[i] = c.W1 + col; wstride[i] = c.K1; xp[i] = c.x1 + col; }
-        } else if (ch < nch1 + nch2) {
-            const int col = (ch - nch1) * kChunk + lane * 8;
-            if (col < c.K2) { wp[i] = c.W2 + col; wstride[i] = c.K2; xp[i] = c.x2 + col; }
-        }
-    }
     bool first = true;
-    half2_t xs[CP][4];
     for (int b0 = r0; b0 < r1; b0 += kRowBatch) {
         const int b1 = (b0 + kRowBatch < r1) ? b0 + kRowBatch : r1;
-        if (wave < kStreamers) {
+        if (streamer && c.K2 > 0) {
+            constexpr int RPI = (16 / CPD) > 0 ? (16 / CPD) : 1;
+            const int nch = (c.K2 + kChunk - 1) / kChunk;
+            // a chunk that does not exist for this lane reads column 0 with a zero activation slice
+            int coff[CPD];
+            bool have[CPD];
+#pragma unroll
+            for (int i = 0; i < CPD; ++i) {
+                const int col = (ks + i * kStreamers) * kChunk + lane * 8;
+                have[i] = (ks + i * kStreamers) < nch && col < c.K2;
+                coff[i] = have[i] ? col : 0;
+            }
             // rows past the batch re-read its last row (no conditional loads, see gemv_tiles)
-            auto load_rows = [&](u32x4 (&w)[RPI][CP], int r) {
+            auto load_rows = [&](u32x4 (&w)[RPI][CPD], int r) {
 #pragma unroll
                 for (int j = 0; j < RPI; ++j) {
                     const int rr = (r + j < b1) ? r + j : b1 - 1;
+                    const half_t* rp = c.W2 + (size_t)rr * (size_t)c.K2;
 #pragma unroll
-                    for (int i = 0; i < CP; ++i) w[j][i] = ld_stream16(wp[i] + (size_t)rr * wstride[i]);
+                    for (int i = 0; i < CPD; ++i) w[j][i] = ld_stream16(rp + coff[i]);
                 }
             };
-            auto finish_rows = [&](const u32x4 (&w)[RPI][CP], int r) {
+            u32x4 wa[RPI][CPD], wb[RPI][CPD];
+            load_rows(wa, b0);
+            if (first) down_ready();
+            half2_t xs[CPD][4];
+#pragma unroll
+            for (int i = 0; i < CPD; ++i) {
+                u32x4 xv = {0u, 0u, 0u, 0u};
+                if (have[i]) xv = ld_agent16(c.x2 + coff[i]);
+                xs[i][0] = as_h2(xv.x); xs[i][1] = as_h2(xv.y); xs[i][2] = as_h2(xv.z); xs[i][3] = as_h2(xv.w);
+            }
+            auto finish_rows = [&](const u32x4 (&w)[RPI][CPD], int r) {
 #pragma unroll
                 for (int j = 0; j < RPI; ++j) {
                     float acc = 0.f;
 #pragma unroll
-                    for (int i = 0; i < CP; ++i) acc = dot8(w[j][i], xs[i], acc);
+                    for (int i = 0; i < CPD; ++i) acc = dot8(w[j][i], xs[i], acc);
                     acc = wave_sum(acc);
-                    if (r + j < b1 && lane == 0) sh.red[r + j - b0][wave] = acc;
+                    if (r + j < b1 && lane == 0) sh.red_down[r + j - b0][ks] = acc;
                 }
             };
-            u32x4 wa[RPI][CP], wb[RPI][CP];
-            load_rows(wa, b0);
-            if (first) {
-                ready();
-#pragma unroll
-                for (int i = 0; i < CP; ++i) {
-                    u32x4 xv = {0u, 0u, 0u, 0u};
-                    if (xp[i]) xv = ld_agent16(xp[i]);
-                    xs[i][0] = as_h2(xv.x); xs[i][1] = as_h2(xv.y); xs[i][2] = as_h2(xv.z); xs[i][3] = as_h2(xv.w);
-                }
-            }
             for (int r = b0; r < b1; r += 2 * RPI) {   // two tiles in flight, branch-free body
                 load_rows(wb, r + RPI);
                 finish_rows(wa, r);
@@ -803,13 +790,51 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        if (o_index >= 0 && c.K1 > 0) {
+            auto load_row = [&](u32x4 (&w)[NCH], int r) {
+                const int rr = r < b1 ? r : b1 - 1;
+                const half_t* rp = c.W1 + (size_t)rr * (size_t)c.K1;
+#pragma unroll
+                for (int i = 0; i < NCH; ++i) {
+                    const int col = i * kChunk + lane * 8;
+                    w[i] = ld_stream16(rp + (col < c.K1 ? col : 0));
+                }
+            };
+            u32x4 wa[NCH], wb[NCH];
+            load_row(wa, b0 + o_index);
+            if (first) o_ready();
+            half2_t xs[NCH][4];
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                const int col = i * kChunk + lane * 8;
+                u32x4 xv = {0u, 0u, 0u, 0u};
+                if (col < c.K1) xv = ld_agent16(c.x1 + col);
+                xs[i][0] = as_h2(xv.x); xs[i][1] = as_h2(xv.y); xs[i][2] = as_h2(xv.z); xs[i][3] = as_h2(xv.w);
+            }
+            auto finish_row = [&](const u32x4 (&w)[NCH], int r) {
+                float acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < NCH; ++i) acc = dot8(w[i], xs[i], acc);
+                acc = wave_sum(acc);
+                if (r < b1 && lane == 0) sh.red_o[r - b0] = acc;
+            };
+            for (int r = b0 + o_index; r < b1; r += 2 * n_o) {
+                load_row(wb, r + n_o);
+                finish_row(wa, r);
+                __builtin_amdgcn_sched_barrier(0);
+                load_row(wa, r + 2 * n_o);
+                finish_row(wb, r + n_o);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
         first = false;
         __syncthreads();
         const int t = threadIdx.x;
         if (t < b1 - b0) {
             const int r = b0 + t;
             float v = 0.f;
-            for (int k = 0; k < kStreamers; ++k) v += sh.red[t][k];
+            if (c.K2 > 0) for (int k = 0; k < kStreamers; ++k) v += sh.red_down[t][k];
+            if (c.K1 > 0) v += sh.red_o[t];
             if (c.bias1) v += (float)c.bias1[r];
             if (c.bias2) v += (float)c.bias2[r];
             if (c.base0) v += (float)c.base0[r];

@@ -95,29 +95,32 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_b(LayerParams p) {
     if (item < p.heads * nsplit) attention_item(p, item / nsplit, item % nsplit, nsplit, S, lane, 0);
 }
 
-template <int CPC>
+template <int NCH, int CPD>
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
     __shared__ StageCShared sh;
+    const int wave = first_lane(threadIdx.x >> 6);
     const StageC c = make_stage_c(p);
-    stage_c_rows<CPC>(c, blockIdx.x, gridDim.x, sh, [] {});
+    stage_c_rows<NCH, CPD>(c, blockIdx.x, gridDim.x, sh, true, wave, wave, kStreamers, [] {}, [] {});
 }
 
 // ---- fused mode: one persistent launch ---------------------------------------------------------
 // One workgroup per compute unit, eight waves: four streaming waves (one per SIMD) and four helper waves.
 //   streaming wave: first QKV tile in flight -> LayerNorm -> its QKV rows -> bump kBarQkv -> its MLP-up
-//                   rows -> bump kBarUp -> (helps with attention items if any are left) -> stage C: first
-//                   weight tile in flight, wait for kBarUp and kBarHeads, O-projection + MLP-down rows,
-//                   row reduction, bias, residual.
+//                   rows -> bump kBarUp -> (helps with attention items if any are left) -> MLP-down rows
+//                   of stage C (first weight tile in flight, then wait for kBarUp).
 //   helper wave:    waits for kBarQkv, then takes (head, split) attention items from the workgroup's
-//                   queue at raised wave priority.  Attention is a chain of dependent memory round
-//                   trips; it runs beside the MLP-up streaming instead of in front of it.
+//                   queue at raised wave priority, then does the O-projection rows of stage C (first
+//                   rows in flight, then wait for kBarHeads).  Attention is a chain of dependent memory
+//                   round trips; it and the O projection run beside the MLP-up / MLP-down streaming
+//                   instead of in front of it.
+//   all waves:      row reduction in LDS, bias, residual.
 // The last workgroup to leave zeroes the counters for the next launch.  All workgroups must be
 // co-resident (the host launches one per compute unit); every wait is bounded.
 struct FusedShared { int attn_next; int arrived[2]; };
 
 __device__ __forceinline__ int lds_take(int* p) { return __hip_atomic_fetch_add(p, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 
-template <int NCH, int CPC, bool EX>
+template <int NCH, int CPD, bool EX>
 __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     __shared__ FusedShared q;
     __shared__ StageCShared shc;
@@ -135,8 +138,7 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     const int S = load_seq_len(p);
     const int nsplit = effective_split(p, S);
     const int nitems = p.heads * nsplit;
-    int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
-    if (p.dbg & 1) attn_count = 0;
+    const int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
     auto take_attention_items = [&] {
         for (;;) {
             int t = 0;
@@ -167,7 +169,7 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
         trace_mark(p, 5);
         event_wait(p.mbox, kBarQkv, status);
         take_attention_items();
-    } else if (!(p.dbg & 2)) {
+    } else {
         event_wait(p.mbox, kBarQkv, status);
         __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
         take_attention_items();
@@ -176,12 +178,11 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     trace_mark(p, 9);
     {
         const StageC c = make_stage_c(p);
-        stage_c_rows<CPC>(c, b, G, shc, [&] {
-            event_wait(p.mbox, kBarUp, status);
-            trace_mark(p, 6);
-            if (!(p.dbg & 1)) event_wait(p.mbox, kBarHeads, status);
-            trace_mark(p, 7);
-        });
+        const bool streamer = wave < kStreamers;
+        stage_c_rows<NCH, CPD>(
+            c, b, G, shc, streamer, wave, streamer ? -1 : wave - kStreamers, kStreamers,
+            [&] { event_wait(p.mbox, kBarUp, status); trace_mark(p, 6); },
+            [&] { event_wait(p.mbox, kBarHeads, status); trace_mark(p, 7); });
     }
     trace_mark(p, 10);
     // the last workgroup to leave re-arms the counters and mailboxes for the next launch
@@ -257,11 +258,12 @@ __global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __res
     }
 }
 
-// token <- argmax, seq_len <- seq_len + 1, history[step] <- token
-__global__ void k_pick_and_advance(const float* __restrict__ best_val, const int* __restrict__ best_idx, int n,
-                                   int* __restrict__ state, int* __restrict__ history, int hist_cap) {
-    __shared__ float sv[256];
-    __shared__ int si[256];
+// token <- argmax, seq_len <- seq_len + 1, history[step] <- token   (one workgroup of 256 threads)
+__global__ __launch_bounds__(256) void k_pick_and_advance(const float* __restrict__ best_val, const int* __restrict__ best_idx,
+                                                          int n, int* __restrict__ state, int* __restrict__ history, int hist_cap) {
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -269,11 +271,17 @@ __global__ void k_pick_and_advance(const float* __restrict__ best_val, const int
         const int r = best_idx[i];
         if (v > bv || (v == bv && r < bi)) { bv = v; bi = r; }
     }
-    sv[threadIdx.x] = bv; si[threadIdx.x] = bi;
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {     // ties go to the lower index, whatever the reduction order
+        const float ov = __shfl_xor(bv, m, kWave);
+        const int oi = __shfl_xor(bi, m, kWave);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int t = 1; t < (int)blockDim.x; ++t)
-            if (sv[t] > bv || (sv[t] == bv && si[t] < bi)) { bv = sv[t]; bi = si[t]; }
+        for (int w = 1; w < 4; ++w)
+            if (sv[w] > bv || (sv[w] == bv && si[w] < bi)) { bv = sv[w]; bi = si[w]; }
         const int step = state[2];
         state[0] = bi;
         state[1] = state[1] + 1;
@@ -361,15 +369,15 @@ int check_dims(const cfpp_neox_dims* d) {
 
 // launch geometry for one set of dims
 struct Plan {
-    int nch;        // 512-half chunks of the hidden row (stage-A registers)
-    int cpc;        // stage-C chunks ([attention | MLP intermediate]) per streaming wave
+    int nch;        // 512-half chunks of the hidden row (stage-A and O-projection registers)
+    int cpd;        // MLP-down chunks per streaming wave
 };
 
 int make_plan(const cfpp_neox_dims& d, Plan* out) {
     Plan p{};
     p.nch = (d.hidden + kChunk - 1) / kChunk;
-    p.cpc = (p.nch + (d.ffn + kChunk - 1) / kChunk + kStreamers - 1) / kStreamers;
-    if (p.nch < 1 || p.nch > 8 || p.cpc < 1 || p.cpc > 10) return CFPP_ERR_DIMS;
+    p.cpd = ((d.ffn + kChunk - 1) / kChunk + kStreamers - 1) / kStreamers;
+    if (p.nch < 1 || p.nch > 8 || p.cpd < 1 || p.cpd > 8) return CFPP_ERR_DIMS;
     *out = p;
     return CFPP_OK;
 }
@@ -392,14 +400,14 @@ int launch_stage_a_t(const LayerParams& p, int grid, hipStream_t st) {
     else hipLaunchKernelGGL((k_stage_a<NCH, false>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
     return launch_check();
 }
-template <int CPC>
+template <int NCH, int CPD>
 int launch_stage_c_t(const LayerParams& p, int grid, hipStream_t st) {
-    hipLaunchKernelGGL((k_stage_c<CPC>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
+    hipLaunchKernelGGL((k_stage_c<NCH, CPD>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
     return launch_check();
 }
-template <int NCH, int CPC>
+template <int NCH, int CPD>
 int launch_fused_t(const LayerParams& p, int grid, hipStream_t st) {
-    const void* fn = p.H == NCH * kChunk ? (const void*)(k_fused<NCH, CPC, true>) : (const void*)(k_fused<NCH, CPC, false>);
+    const void* fn = p.H == NCH * kChunk ? (const void*)(k_fused<NCH, CPD, true>) : (const void*)(k_fused<NCH, CPD, false>);
     static int coop = env_int("CFPP_COOPERATIVE", 0);
     LayerParams pp = p;
     void* args[] = {&pp};
@@ -409,9 +417,10 @@ int launch_fused_t(const LayerParams& p, int grid, hipStream_t st) {
 }
 
 #define CFPP_NCH_CASES(X) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8)
-// (hidden chunks, stage-C chunks per streaming wave) of the Pythia family, ffn = 4 hidden:
-// 512 -> (1,2), 768/1024 -> (2,3), 2048 -> (4,5), 2560 -> (5,7), 4096 -> (8,10); (8,8) is 4096 with ffn 11008
-#define CFPP_SHAPE_CASES(X) X(1, 2) X(2, 3) X(4, 5) X(5, 7) X(8, 10) X(8, 8)
+// (hidden chunks, MLP-down chunks per streaming wave).  The Pythia family has ffn = 4 hidden, so both
+// numbers coincide: 512 -> (1,1), 768/1024 -> (2,2), 2048 -> (4,4), 2560 -> (5,5), 4096 -> (8,8);
+// (8,6) is hidden 4096 with ffn 11008
+#define CFPP_SHAPE_CASES(X) X(1, 1) X(2, 2) X(4, 4) X(5, 5) X(8, 8) X(8, 6)
 
 int launch_stage_a(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
     switch (pl.nch) {
@@ -422,19 +431,19 @@ int launch_stage_a(const Plan& pl, const LayerParams& p, int grid, hipStream_t s
     return CFPP_ERR_DIMS;
 }
 int launch_stage_c(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
-#define X(a, b) if (pl.nch == a && pl.cpc == b) return launch_stage_c_t<b>(p, grid, st);
+#define X(a, b) if (pl.nch == a && pl.cpd == b) return launch_stage_c_t<a, b>(p, grid, st);
     CFPP_SHAPE_CASES(X)
 #undef X
     return CFPP_ERR_DIMS;
 }
 int launch_fused(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
-#define X(a, b) if (pl.nch == a && pl.cpc == b) return launch_fused_t<a, b>(p, grid, st);
+#define X(a, b) if (pl.nch == a && pl.cpd == b) return launch_fused_t<a, b>(p, grid, st);
     CFPP_SHAPE_CASES(X)
 #undef X
     return CFPP_ERR_DIMS;
 }
 bool shape_supported(const Plan& pl) {
-#define X(a, b) if (pl.nch == a && pl.cpc == b) return true;
+#define X(a, b) if (pl.nch == a && pl.cpd == b) return true;
     CFPP_SHAPE_CASES(X)
 #undef X
     return false;
@@ -501,7 +510,6 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     p.mbox = reinterpret_cast<int*>(ws + L.mbox);
     p.c_base0 = p.x; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 1;
     p.trace = g_trace;
-    p.dbg = env_int("CFPP_DBG", 0);
     *out = p;
     return CFPP_OK;
 }
