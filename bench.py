@@ -144,6 +144,14 @@ def main():
     torch.cuda.synchronize()
     log(f"[bench] built {args.model} ({cfg.n_layers} layers) in {time.perf_counter() - t0:.1f} s; cache rows {rows}")
 
+    # a plain device-to-device copy of known size (256 MiB read + 256 MiB written): the reference point
+    # that hardware-counter runs (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) are scaled by
+    cal_src = torch.empty(128 << 20, dtype=torch.float16, device=dev).normal_()
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    torch.cuda.synchronize()
+    del cal_src, cal_dst
+
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         dec.set_state(11, args.ctx)
