@@ -397,6 +397,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     DEFINE_MODEL_OPS(m, pythia_2b8)
     DEFINE_MODEL_OPS(m, pythia_6b9)
 
+    // any supported GPT-NeoX geometry (other Pythia sizes): same tensor arguments as the per-model ops
+    m.def("neox_decoder_layer", [](int64_t hidden, int64_t heads, int64_t head_dim, int64_t rotary_dim, int64_t ffn, double eps,
+                                   bool split, LAYER_ARGS, Tensor mlp_down_weight, Tensor mlp_down_bias, int64_t current_seq_len) {
+        const Model m{"neox_decoder_layer", 2,
+                      {(int32_t)hidden, (int32_t)heads, (int32_t)head_dim, (int32_t)rotary_dim, (int32_t)ffn, (float)eps}};
+        TORCH_CHECK(cfpp_neox_workspace_bytes(&m.dims) > 0, "unsupported layer dimensions");
+        return decoder_layer(m, split ? CFPP_MODE_SPLIT : CFPP_MODE_FUSED, LAYER_PACK(mlp_down_weight, mlp_down_bias), current_seq_len);
+    });
     m.def("cfpp_version", []() { return std::string(cfpp_version()); });
     m.def("debug_set_trace", [](c10::optional<Tensor> buf) {
         // int64 device tensor of at least 1024*16*16 elements, or None to switch tracing off

@@ -1,0 +1,48 @@
+"""Writes the golden fixtures of the decode-step parity tests.
+
+The reference repository holds no stored expected outputs (its scripts compute them live on a CUDA device),
+so the fixtures are produced by this repository's CPU oracle after it has been pinned against HuggingFace
+GPTNeoXLayer, a brute-force loop and closed forms (tests/test_oracle_pins.py).  Inputs are regenerated from
+fixed seeds (oracle.neox_oracle.make_layer_weights / make_layer_inputs); only the expected outputs are
+stored, as float32 in one .npz per case.
+
+    python tests/golden/make_golden.py
+"""
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+from oracle import neox_oracle as O  # noqa: E402
+
+CASES = {
+    # name: (dims, seq_len, seed)
+    "neox_h512_s37": (O.NeoxDims(hidden=512, heads=8, head_dim=64, rotary_dim=16, ffn=2048), 37, 101),
+    "pythia_2b8_s512": (O.PYTHIA_2B8, 512, 102),
+    "pythia_6b9_s2048": (O.PYTHIA_6B9, 2048, 103),
+}
+
+
+def inputs(name):
+    dims, S, seed = CASES[name]
+    w = O.make_layer_weights(dims, layer=seed)
+    x, k, v, cos, sin = O.make_layer_inputs(dims, S, capacity=S + 1, seed=seed)
+    return dims, S, w, x, k, v, cos, sin
+
+
+def main():
+    torch.set_num_threads(max(1, os.cpu_count() or 1))
+    for name in CASES:
+        dims, S, w, x, k, v, cos, sin = inputs(name)
+        r = O.neox_layer_decode(x, w, k, v, cos, sin, S, dims, dtype=torch.float64, round_io=True)
+        out = {n: r[n].to(torch.float32).numpy() for n in ("output", "k_new", "v_new", "attn_output", "mlp_intermediate")}
+        path = os.path.join(HERE, name + ".npz")
+        np.savez_compressed(path, **out)
+        print(name, {n: a.shape for n, a in out.items()}, os.path.getsize(path), "bytes")
+
+
+if __name__ == "__main__":
+    main()
