@@ -447,41 +447,52 @@ __device__ __forceinline__ void finish_row_tile(const RowTile<NCH, RPI>& t, cons
 // Tiles t = 0 .. ntiles-1 of one wave: tile t covers rows row_of(t) + j*stride_in_tile, j < RPI (rows >=
 // nrows do not exist).  Two tiles are in flight: the loads of the next tile are issued before the current
 // one is reduced.  `pre` already holds the loads of tile 0 (issued by the caller before something slow:
-// the LayerNorm prologue or a barrier).  The loop body is free of branches: the loads of a tile past the
-// end re-read the last tile instead of being skipped, because a conditional load makes the compiler's
-// wait-count bookkeeping assume the shorter path and drain the pipeline at every tile.
+// the LayerNorm prologue or a barrier).  The loop body is free of branches, because a conditional load
+// makes the compiler's wait-count bookkeeping assume the shorter path and drain the pipeline at every
+// tile; the last one or two tiles of a segment are peeled off behind the loop instead, so that no tile is
+// ever loaded twice.
 // The tiles are processed in segments of kParkRows rows; `flush(park, first_index)` runs after each
-// segment, outside the streaming loop (no global store may sit inside it, see RowPark); parked value k
-// (counting from first_index) belongs to the k-th row this wave finished.
+// segment, outside the streaming loop (no global store may sit inside it, see RowPark), with the first
+// tile of the next segment already in flight; parked value k (counting from first_index) belongs to the
+// k-th row this wave finished.
 template <int NCH, int RPI, bool EXACT, class RowOf, class Flush>
 __device__ __forceinline__ void gemv_tiles(const half_t* __restrict__ W, int K, int nrows, int stride_in_tile, int ntiles,
                                            RowOf&& row_of, const half2_t (&x)[NCH][4], int lane, RowTile<NCH, RPI>& pre,
                                            RowPark& park, Flush&& flush) {
     constexpr int kSegTiles = (kParkRows / RPI) & ~1;   // even, so a segment is a whole number of loop trips
     static_assert(kSegTiles >= 2, "tile larger than the park");
-    auto valid_rows = [&](int t) {
+    auto valid_rows = [&](int t) {   // only the last tile of a wave can be short
         int v = 0;
-        if (t < ntiles) {
-            const int r = row_of(t);
+        const int r = row_of(t);
 #pragma unroll
-            for (int j = 0; j < RPI; ++j) v += (r + j * stride_in_tile < nrows) ? 1 : 0;
-        }
+        for (int j = 0; j < RPI; ++j) v += (r + j * stride_in_tile < nrows) ? 1 : 0;
         return v;
     };
-    auto tile_row = [&](int t) { return row_of(t < ntiles ? t : ntiles - 1); };
+    auto load = [&](RowTile<NCH, RPI>& t, int i) { load_row_tile<NCH, RPI, EXACT>(t, W, K, row_of(i), stride_in_tile, nrows, lane); };
     int done = 0;
     for (int seg = 0; seg < ntiles; seg += kSegTiles) {
         const int seg_end = seg + kSegTiles < ntiles ? seg + kSegTiles : ntiles;
-        if (seg != 0) load_row_tile<NCH, RPI, EXACT>(pre, W, K, tile_row(seg), stride_in_tile, nrows, lane);
         RowTile<NCH, RPI> other;
-        for (int t = seg; t < seg_end; t += 2) {
-            load_row_tile<NCH, RPI, EXACT>(other, W, K, tile_row(t + 1), stride_in_tile, nrows, lane);
-            finish_row_tile<NCH, RPI>(pre, x, valid_rows(t), lane, park);
+        int t = seg;
+        for (; t + 2 < seg_end; t += 2) {     // tiles t+1 and t+2 exist and are full
+            load(other, t + 1);
+            finish_row_tile<NCH, RPI>(pre, x, RPI, lane, park);
             __builtin_amdgcn_sched_barrier(0);   // a third tile's loads must not be scheduled above this point
-            load_row_tile<NCH, RPI, EXACT>(pre, W, K, tile_row(t + 2), stride_in_tile, nrows, lane);
-            finish_row_tile<NCH, RPI>(other, x, t + 1 < seg_end ? valid_rows(t + 1) : 0, lane, park);
+            load(pre, t + 2);
+            finish_row_tile<NCH, RPI>(other, x, RPI, lane, park);
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (t + 1 < seg_end) {
+            load(other, t + 1);
+            finish_row_tile<NCH, RPI>(pre, x, RPI, lane, park);
+            __builtin_amdgcn_sched_barrier(0);
+            if (seg_end < ntiles) load(pre, seg_end);
+            finish_row_tile<NCH, RPI>(other, x, valid_rows(t + 1), lane, park);
+        } else {
+            finish_row_tile<NCH, RPI>(pre, x, valid_rows(t), lane, park);
+            if (seg_end < ntiles) load(pre, seg_end);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         flush(park, done);
         done += park.n;
         park.n = 0;
@@ -781,13 +792,21 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
                     if (r + j < b1 && lane == 0) sh.red_down[r + j - b0][ks] = acc;
                 }
             };
-            for (int r = b0; r < b1; r += 2 * RPI) {   // two tiles in flight, branch-free body
+            int r = b0;
+            for (; r + 2 * RPI < b1; r += 2 * RPI) {   // two tiles in flight, branch-free body, tail peeled
                 load_rows(wb, r + RPI);
                 finish_rows(wa, r);
                 __builtin_amdgcn_sched_barrier(0);   // a third tile's loads must not be scheduled above this point
                 load_rows(wa, r + 2 * RPI);
                 finish_rows(wb, r + RPI);
                 __builtin_amdgcn_sched_barrier(0);
+            }
+            if (r + RPI < b1) {
+                load_rows(wb, r + RPI);
+                finish_rows(wa, r);
+                finish_rows(wb, r + RPI);
+            } else {
+                finish_rows(wa, r);
             }
         }
         if (o_index >= 0 && c.K1 > 0) {
@@ -818,13 +837,21 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
                 acc = wave_sum(acc);
                 if (r < b1 && lane == 0) sh.red_o[r - b0] = acc;
             };
-            for (int r = b0 + o_index; r < b1; r += 2 * n_o) {
+            int r = b0 + o_index;
+            for (; r + 2 * n_o < b1; r += 2 * n_o) {
                 load_row(wb, r + n_o);
                 finish_row(wa, r);
                 __builtin_amdgcn_sched_barrier(0);
                 load_row(wa, r + 2 * n_o);
                 finish_row(wb, r + n_o);
                 __builtin_amdgcn_sched_barrier(0);
+            }
+            if (r + n_o < b1) {
+                load_row(wb, r + n_o);
+                finish_row(wa, r);
+                finish_row(wb, r + n_o);
+            } else if (r < b1) {
+                finish_row(wa, r);
             }
         }
         first = false;
