@@ -37,7 +37,9 @@ constexpr int kMaxSplit = 64;          // KV splits per head (upper bound; the e
 constexpr int kSplitRows = 64;         // target cache rows per (head, split) item
 constexpr int kMaxWaves = 16;          // waves per workgroup
 constexpr int kRowBatch = 32;          // stage-C rows per workgroup pass
-constexpr int kUpRpi = 2;              // MLP-up rows per dynamically scheduled task
+constexpr int kUpRpi = 2;              // adjacent MLP-up rows per tile
+constexpr int kStreamers = 4;          // streaming waves per workgroup: one per SIMD of the compute unit
+constexpr int kUpPhases = 2;           // the MLP intermediate is produced and consumed in this many phases
 constexpr float kNegBig = -1.0e30f;
 constexpr int kSpinLimit = 1 << 20;    // bounded device-side waits (order of a second)
 
@@ -45,10 +47,10 @@ enum : int { kStatusSpin = 1, kStatusSeq = 2 };
 // counters in LayerParams::bar (self-resetting: the last workgroup to leave zeroes them)
 enum BarSlot : int {
     kBarQkv = 0,      // streaming waves that have written their QKV rows
-    kBarUp = 1,       // streaming waves that have written their MLP-up rows
-    kBarHeads = 2,    // heads whose attention output is merged
-    kBarExit = 3,     // workgroups that have finished
-    kBarStatus = 4    // failure flags (kStatusSpin, kStatusSeq); not reset by the kernels
+    kBarUp = 1,       // kBarUp + g: streaming waves that have written their MLP-up rows of phase g (kUpPhases slots)
+    kBarHeads = 3,    // heads whose attention output is merged
+    kBarExit = 4,     // workgroups that have finished
+    kBarStatus = 5    // failure flags (kStatusSpin, kStatusSeq); not reset by the kernels
 };
 
 struct LayerParams {
@@ -63,6 +65,7 @@ struct LayerParams {
     int seq_len;
     const int* d_seq_len;
     int max_split;      // cap on the KV splits per head (<= kMaxSplit)
+    int row_walk_strided;   // streaming waves take interleaved instead of contiguous row ranges
     // scratch
     float* qkv_raw;     // [3H] fp32: W_qkv ln1(x) + b_qkv, before RoPE
     half_t* attn_vec;   // [H] fp16: merged attention output (input of the O projection)
@@ -292,97 +295,117 @@ __device__ __forceinline__ int effective_split(const LayerParams& p, int S) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// stage A: LayerNorm into registers, then row-per-wave streaming GEMV
+// stage A: LayerNorm shared by the workgroup, then row-per-wave streaming GEMV
 // ------------------------------------------------------------------------------------------------
-// Every wave loads the whole input row (lane l holds columns i*512 + 8l .. +8 of every chunk i),
-// computes mean and variance two-pass in fp32 and keeps the normalised, affine-transformed row as
-// packed fp16.  The post-attention LayerNorm (input of the MLP) shares the statistics with the input
-// LayerNorm because the residual is parallel (reference include/5090/pythia_2b8/kernel.cuh:811-818):
-// ln_affine() re-reads x (8 KB, cache resident) with the saved statistics when that variant is needed,
-// so only one variant is live at a time.  x stays packed and is unpacked per pass (register budget).
-struct LnStats { float mean, rstd; };
-
-// Compiler-only barrier on a packed register: stops common-subexpression elimination from keeping the
-// fp32 expansion of x alive across the LayerNorm passes (it emits no instruction).
-__device__ __forceinline__ void keep_packed(u32x4& v) {
-    asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
-}
-
+// The NW waves of a workgroup split the input row into 512-half chunks (chunk i belongs to wave i % NW):
+// a wave loads its chunks of x and of the affine vectors, the chunk sums meet in LDS (mean, then
+// variance, two-pass, fp32; chunk partials are added in chunk order, so the result does not depend on
+// NW), and the normalised rows are left in LDS as packed fp16: slot 0 with the input LayerNorm's affine
+// transform, slot 1 (if TWO) with the post-attention LayerNorm's, which shares the statistics because
+// the residual is parallel (reference include/5090/pythia_2b8/kernel.cuh:811-818).  Every streaming wave
+// then copies the row it needs into registers (lane l holds columns i*512 + 8l .. +8 of every chunk i;
+// columns >= H are zero).  Letting every wave load the whole row itself makes a thousand waves ask for
+// the same few cache lines at the same moment, which costs several microseconds at the start of a launch.
 template <int NCH>
-__device__ __forceinline__ void ln_apply(const u32x4 (&rx)[NCH], const u32x4 (&rw)[NCH], const u32x4 (&rb)[NCH], int H,
-                                         LnStats st, int lane, half2_t (&dst)[NCH][4]) {
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        const bool in = i * kChunk + lane * 8 < H;
-        float xv[8], g[8], b[8], y[8];
-        unpack8(rx[i], xv); unpack8(rw[i], g); unpack8(rb[i], b);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) y[j] = in ? (xv[j] - st.mean) * st.rstd * g[j] + b[j] : 0.f;
-        const u32x4 pk = pack8(y);
-        dst[i][0] = as_h2(pk.x); dst[i][1] = as_h2(pk.y); dst[i][2] = as_h2(pk.z); dst[i][3] = as_h2(pk.w);
-    }
-}
+struct LnShared {
+    float part[2][NCH];
+    __attribute__((aligned(16))) half_t y[2][NCH * kChunk];
+};
+template <int NCH, int NW>
+struct LnOwn {
+    static constexpr int OWN = (NCH + NW - 1) / NW;
+    u32x4 rx[OWN], rw1[OWN], rb1[OWN], rw2[OWN], rb2[OWN];
+};
 
-template <int NCH>
-__device__ __forceinline__ void ln_load3(const half_t* __restrict__ x, const half_t* __restrict__ w,
-                                         const half_t* __restrict__ b, int H, int lane, u32x4 (&rx)[NCH],
-                                         u32x4 (&rw)[NCH], u32x4 (&rb)[NCH]) {
+template <int NCH, int NW, bool TWO>
+__device__ __forceinline__ void ln_coop_load(LnOwn<NCH, NW>& o, const half_t* __restrict__ x, int H,
+                                             const half_t* __restrict__ w1, const half_t* __restrict__ b1,
+                                             const half_t* __restrict__ w2, const half_t* __restrict__ b2, int wave, int lane) {
     const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        const int col = i * kChunk + lane * 8;
-        const bool in = col < H;
-        rx[i] = in ? ld16(x + col) : z;
-        rw[i] = in ? ld16(w + col) : z;
-        rb[i] = in ? ld16(b + col) : z;
-    }
-}
-
-template <int NCH>
-__device__ __forceinline__ LnStats ln_first(const half_t* __restrict__ x, int H, float eps, const half_t* __restrict__ w,
-                                            const half_t* __restrict__ b, int lane, half2_t (&dst)[NCH][4]) {
-    // x and the affine vectors are requested together: one memory round trip for the prologue
-    u32x4 rx[NCH], rw[NCH], rb[NCH];
-    ln_load3<NCH>(x, w, b, H, lane, rx, rw, rb);
-    float s = 0.f;
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        float xv[8];
-        unpack8(rx[i], xv);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) s += xv[j];
-    }
-    LnStats st;
-    st.mean = wave_sum(s) / (float)H;
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) keep_packed(rx[i]);
-    float q = 0.f;
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        if (i * kChunk + lane * 8 < H) {
-            float xv[8];
-            unpack8(rx[i], xv);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) { const float d = xv[j] - st.mean; q += d * d; }
+    for (int k = 0; k < LnOwn<NCH, NW>::OWN; ++k) {
+        const int col = (wave + k * NW) * kChunk + lane * 8;
+        const bool in = wave + k * NW < NCH && col < H;
+        o.rx[k] = in ? ld16(x + col) : z;
+        o.rw1[k] = in ? ld16(w1 + col) : z;
+        o.rb1[k] = in ? ld16(b1 + col) : z;
+        if (TWO) {
+            o.rw2[k] = in ? ld16(w2 + col) : z;
+            o.rb2[k] = in ? ld16(b2 + col) : z;
         }
     }
-    st.rstd = 1.0f / sqrtf(wave_sum(q) / (float)H + eps);
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) keep_packed(rx[i]);
-    ln_apply<NCH>(rx, rw, rb, H, st, lane, dst);
-    // keep later weight loads from being scheduled up into the prologue (they would only add register pressure)
-    __builtin_amdgcn_sched_barrier(0);
-    return st;
 }
 
+// Every wave of the workgroup must call this (workgroup barriers inside).
+template <int NCH, int NW, bool TWO>
+__device__ __forceinline__ void ln_coop_finish(const LnOwn<NCH, NW>& o, int H, float eps, LnShared<NCH>& sh, int wave, int lane) {
+    constexpr int OWN = LnOwn<NCH, NW>::OWN;
+#pragma unroll
+    for (int k = 0; k < OWN; ++k) {
+        const int i = wave + k * NW;
+        if (i < NCH) {
+            float xv[8], s = 0.f;
+            unpack8(o.rx[k], xv);     // lanes past H hold zeros
+#pragma unroll
+            for (int j = 0; j < 8; ++j) s += xv[j];
+            s = wave_sum(s);
+            if (lane == 0) sh.part[0][i] = s;
+        }
+    }
+    __syncthreads();
+    float mean = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) mean += sh.part[0][i];
+    mean /= (float)H;
+#pragma unroll
+    for (int k = 0; k < OWN; ++k) {
+        const int i = wave + k * NW;
+        if (i < NCH) {
+            float xv[8], q = 0.f;
+            unpack8(o.rx[k], xv);
+            if (i * kChunk + lane * 8 < H) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) { const float d = xv[j] - mean; q += d * d; }
+            }
+            q = wave_sum(q);
+            if (lane == 0) sh.part[1][i] = q;
+        }
+    }
+    __syncthreads();
+    float var = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) var += sh.part[1][i];
+    const float rstd = 1.0f / sqrtf(var / (float)H + eps);
+#pragma unroll
+    for (int k = 0; k < OWN; ++k) {
+        const int i = wave + k * NW;
+        if (i < NCH) {
+            const bool in = i * kChunk + lane * 8 < H;
+            float xv[8], g[8], b[8], y[8];
+            unpack8(o.rx[k], xv); unpack8(o.rw1[k], g); unpack8(o.rb1[k], b);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) y[j] = in ? (xv[j] - mean) * rstd * g[j] + b[j] : 0.f;
+            *reinterpret_cast<u32x4*>(&sh.y[0][i * kChunk + lane * 8]) = pack8(y);
+            if (TWO) {
+                unpack8(o.rw2[k], g); unpack8(o.rb2[k], b);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) y[j] = in ? (xv[j] - mean) * rstd * g[j] + b[j] : 0.f;
+                *reinterpret_cast<u32x4*>(&sh.y[1][i * kChunk + lane * 8]) = pack8(y);
+            }
+        }
+    }
+    __syncthreads();
+}
+
+// The normalised row of slot `which`, into the registers of this wave.
 template <int NCH>
-__device__ __forceinline__ void ln_affine(const half_t* __restrict__ x, int H, LnStats st, const half_t* __restrict__ w,
-                                          const half_t* __restrict__ b, int lane, half2_t (&dst)[NCH][4]) {
-    __builtin_amdgcn_sched_barrier(0);
-    u32x4 rx[NCH], rw[NCH], rb[NCH];
-    ln_load3<NCH>(x, w, b, H, lane, rx, rw, rb);
-    ln_apply<NCH>(rx, rw, rb, H, st, lane, dst);
-    __builtin_amdgcn_sched_barrier(0);
+__device__ __forceinline__ void ln_fetch(const LnShared<NCH>& sh, int which, int lane, half2_t (&dst)[NCH][4]) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(&sh.y[which][i * kChunk + lane * 8]);
+        dst[i][0] = as_h2(v.x); dst[i][1] = as_h2(v.y); dst[i][2] = as_h2(v.z); dst[i][3] = as_h2(v.w);
+    }
+    __builtin_amdgcn_sched_barrier(0);   // keep later weight loads from being scheduled above this point
 }
 
 // RPI weight rows of K = up to NCH*512 halfs held in registers.
@@ -724,10 +747,99 @@ __device__ __forceinline__ StageC make_stage_c(const LayerParams& p) {
     return c;
 }
 
-constexpr int kStreamers = 4;          // streaming waves per workgroup: one per SIMD of the compute unit
+// The MLP-down pass splits K over the kStreamers streaming waves of a workgroup: wave ks owns the 512-half
+// chunks ks, ks + kStreamers, ... ("chunk slots" 0 .. CPD-1 of that wave).  The slots are grouped into
+// kUpPhases phases; phase g needs the MLP intermediate only up to up_phase_rows(CPD, g, F), so it can
+// start as soon as every MLP-up row below that bound is written, while slower workgroups are still
+// busy with the rows above it.
+__host__ __device__ constexpr int down_slot_end(int cpd, int g) { return ((g + 1) * cpd + kUpPhases - 1) / kUpPhases; }
+__host__ __device__ constexpr int down_slot_begin(int cpd, int g) { return g == 0 ? 0 : down_slot_end(cpd, g - 1); }
+__device__ __forceinline__ int up_phase_rows(int cpd, int g, int F) {
+    const int r = down_slot_end(cpd, g) * kStreamers * kChunk;
+    return (g == kUpPhases - 1 || r > F) ? F : r;
+}
+
 struct StageCShared {
-    float red_down[kRowBatch][kStreamers];   // MLP-down partials of the K slices
-    float red_o[kRowBatch];                  // O-projection dot products
+    float red_down[kUpPhases][kRowBatch][kStreamers];   // MLP-down partials per phase and K slice
+    float red_o[kRowBatch];                             // O-projection dot products
+};
+
+// One phase (chunk slots LO .. HI-1) of the MLP-down rows [b0, b1) of a streaming wave.
+template <int LO, int HI>
+struct DownPhase {
+    static constexpr int N = HI - LO;
+    static constexpr int RPI = N > 0 ? ((16 / N) > 0 ? (16 / N) : 1) : 1;
+    static constexpr int NA = N > 0 ? N : 1;
+    typedef u32x4 Tile[RPI][NA];
+
+    // a chunk that does not exist for this lane reads column 0 with a zero activation slice
+    static __device__ __forceinline__ int col_of(const StageC& c, int ks, int lane, int i, bool& have) {
+        const int nch = (c.K2 + kChunk - 1) / kChunk;
+        const int chunk = ks + (LO + i) * kStreamers;
+        const int col = chunk * kChunk + lane * 8;
+        have = chunk < nch && col < c.K2;
+        return have ? col : 0;
+    }
+    // rows past the batch re-read its last row (no conditional loads, see gemv_tiles)
+    static __device__ __forceinline__ void load(const StageC& c, int ks, int lane, Tile& w, int r, int b1) {
+#pragma unroll
+        for (int j = 0; j < RPI; ++j) {
+            const int rr = (r + j < b1) ? r + j : b1 - 1;
+            const half_t* rp = c.W2 + (size_t)rr * (size_t)c.K2;
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                bool have;
+                w[j][i] = ld_stream16(rp + col_of(c, ks, lane, i, have));
+            }
+        }
+    }
+    // `wa` holds the loads of the first tile; ready() runs before the activations are read; next() runs
+    // once the last tile of this phase has been requested (the caller requests the next phase's first tile).
+    template <class Ready, class Next>
+    static __device__ __forceinline__ void run(const StageC& c, int ks, int lane, int b0, int b1, float (*red)[kStreamers],
+                                               Tile& wa, Ready&& ready, Next&& next) {
+        ready();
+        half2_t xs[NA][4];
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            bool have;
+            const int col = col_of(c, ks, lane, i, have);
+            u32x4 xv = {0u, 0u, 0u, 0u};
+            if (have) xv = ld_agent16(c.x2 + col);
+            xs[i][0] = as_h2(xv.x); xs[i][1] = as_h2(xv.y); xs[i][2] = as_h2(xv.z); xs[i][3] = as_h2(xv.w);
+        }
+        auto finish = [&](const Tile& w, int r) {
+#pragma unroll
+            for (int j = 0; j < RPI; ++j) {
+                float acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < N; ++i) acc = dot8(w[j][i], xs[i], acc);
+                acc = wave_sum(acc);
+                if (r + j < b1 && lane == 0) red[r + j - b0][ks] = acc;
+            }
+        };
+        Tile wb;
+        int r = b0;
+        for (; r + 2 * RPI < b1; r += 2 * RPI) {   // two tiles in flight, branch-free body, tail peeled
+            load(c, ks, lane, wb, r + RPI, b1);
+            finish(wa, r);
+            __builtin_amdgcn_sched_barrier(0);   // a third tile's loads must not be scheduled above this point
+            load(c, ks, lane, wa, r + 2 * RPI, b1);
+            finish(wb, r + RPI);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (r + RPI < b1) {
+            load(c, ks, lane, wb, r + RPI, b1);
+            finish(wa, r);
+            __builtin_amdgcn_sched_barrier(0);
+            next();
+            finish(wb, r + RPI);
+        } else {
+            next();
+            finish(wa, r);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
 };
 
 // Stage C for the rows of workgroup `wg`, as two independent GEMVs whose results meet in LDS:
@@ -738,7 +850,7 @@ struct StageCShared {
 //              the whole attention vector in registers (K1 <= NCH*512), two rows in flight; red_o.
 // In the fused kernel the streaming waves do the MLP-down part and the helper waves the O projection,
 // so the attention output is not needed until the (longer) MLP-down pass is over; in split mode the same
-// four waves do one after the other.  `down_ready()` / `o_ready()` run after the first loads of a pass are
+// four waves do one after the other.  `down_ready(g)` / `o_ready()` run after the first loads of a pass (of phase g) are
 // in flight and before its activations are read (the fused kernel waits for the producing event there).
 // The partials are added in a fixed order with the biases and residual terms: deterministic, and
 // identical in both modes.  Every wave of the workgroup must call this (workgroup barriers inside).
@@ -751,62 +863,18 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
     for (int b0 = r0; b0 < r1; b0 += kRowBatch) {
         const int b1 = (b0 + kRowBatch < r1) ? b0 + kRowBatch : r1;
         if (streamer && c.K2 > 0) {
-            constexpr int RPI = (16 / CPD) > 0 ? (16 / CPD) : 1;
-            const int nch = (c.K2 + kChunk - 1) / kChunk;
-            // a chunk that does not exist for this lane reads column 0 with a zero activation slice
-            int coff[CPD];
-            bool have[CPD];
-#pragma unroll
-            for (int i = 0; i < CPD; ++i) {
-                const int col = (ks + i * kStreamers) * kChunk + lane * 8;
-                have[i] = (ks + i * kStreamers) < nch && col < c.K2;
-                coff[i] = have[i] ? col : 0;
-            }
-            // rows past the batch re-read its last row (no conditional loads, see gemv_tiles)
-            auto load_rows = [&](u32x4 (&w)[RPI][CPD], int r) {
-#pragma unroll
-                for (int j = 0; j < RPI; ++j) {
-                    const int rr = (r + j < b1) ? r + j : b1 - 1;
-                    const half_t* rp = c.W2 + (size_t)rr * (size_t)c.K2;
-#pragma unroll
-                    for (int i = 0; i < CPD; ++i) w[j][i] = ld_stream16(rp + coff[i]);
-                }
-            };
-            u32x4 wa[RPI][CPD], wb[RPI][CPD];
-            load_rows(wa, b0);
-            if (first) down_ready();
-            half2_t xs[CPD][4];
-#pragma unroll
-            for (int i = 0; i < CPD; ++i) {
-                u32x4 xv = {0u, 0u, 0u, 0u};
-                if (have[i]) xv = ld_agent16(c.x2 + coff[i]);
-                xs[i][0] = as_h2(xv.x); xs[i][1] = as_h2(xv.y); xs[i][2] = as_h2(xv.z); xs[i][3] = as_h2(xv.w);
-            }
-            auto finish_rows = [&](const u32x4 (&w)[RPI][CPD], int r) {
-#pragma unroll
-                for (int j = 0; j < RPI; ++j) {
-                    float acc = 0.f;
-#pragma unroll
-                    for (int i = 0; i < CPD; ++i) acc = dot8(w[j][i], xs[i], acc);
-                    acc = wave_sum(acc);
-                    if (r + j < b1 && lane == 0) sh.red_down[r + j - b0][ks] = acc;
-                }
-            };
-            int r = b0;
-            for (; r + 2 * RPI < b1; r += 2 * RPI) {   // two tiles in flight, branch-free body, tail peeled
-                load_rows(wb, r + RPI);
-                finish_rows(wa, r);
-                __builtin_amdgcn_sched_barrier(0);   // a third tile's loads must not be scheduled above this point
-                load_rows(wa, r + 2 * RPI);
-                finish_rows(wb, r + RPI);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (r + RPI < b1) {
-                load_rows(wb, r + RPI);
-                finish_rows(wa, r);
-                finish_rows(wb, r + RPI);
+            static_assert(kUpPhases == 2, "two phases are written out below");
+            typedef DownPhase<down_slot_begin(CPD, 0), down_slot_end(CPD, 0)> P0;
+            typedef DownPhase<down_slot_begin(CPD, 1), down_slot_end(CPD, 1)> P1;
+            typename P0::Tile t0;
+            P0::load(c, ks, lane, t0, b0, b1);
+            if constexpr (P1::N > 0) {
+                typename P1::Tile t1;
+                P0::run(c, ks, lane, b0, b1, sh.red_down[0], t0, [&] { if (first) down_ready(0); }, [] {});
+                P1::load(c, ks, lane, t1, b0, b1);
+                P1::run(c, ks, lane, b0, b1, sh.red_down[1], t1, [&] { if (first) down_ready(1); }, [] {});
             } else {
-                finish_rows(wa, r);
+                P0::run(c, ks, lane, b0, b1, sh.red_down[0], t0, [&] { if (first) { down_ready(0); down_ready(1); } }, [] {});
             }
         }
         if (o_index >= 0 && c.K1 > 0) {
@@ -860,7 +928,13 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
         if (t < b1 - b0) {
             const int r = b0 + t;
             float v = 0.f;
-            if (c.K2 > 0) for (int k = 0; k < kStreamers; ++k) v += sh.red_down[t][k];
+            if (c.K2 > 0) {
+#pragma unroll
+                for (int g = 0; g < kUpPhases; ++g) {
+                    if (down_slot_end(CPD, g) > down_slot_begin(CPD, g))
+                        for (int k = 0; k < kStreamers; ++k) v += sh.red_down[g][t][k];
+                }
+            }
             if (c.K1 > 0) v += sh.red_o[t];
             if (c.bias1) v += (float)c.bias1[r];
             if (c.bias2) v += (float)c.bias2[r];

@@ -24,45 +24,66 @@ namespace {
 // EX (hidden == NCH*512) is a template parameter of every kernel, chosen by the host: a run-time branch
 // between the two variants makes the compiler keep two copies of the in-flight tiles.
 
-// QKV rows of one streaming wave: rows first, first+stride, ...; result = dot + bias as raw fp32.
+// The rows a streaming wave takes from a row range [lo, hi) shared by `nw` waves, as tiles of RPI rows:
+// tile t covers rows first + t*step + j*sit, j < RPI, below `end`.
+//   blocked  (default): wave w owns the contiguous rows lo + [w n / nw, (w+1) n / nw) in units of RPI
+//            rows; it walks through memory sequentially, so it meets every memory channel and page in
+//            turn and channel conflicts average out within the wave.
+//   strided: wave w owns tiles w, w + nw, ...; every access of a wave is nw*RPI rows from the last one.
+struct RowWalk { int first, step, sit, end, ntiles; };
+template <int RPI>
+__device__ __forceinline__ RowWalk row_walk(bool strided, int w, int nw, int lo, int hi) {
+    const int units = (hi - lo + RPI - 1) / RPI;
+    RowWalk rw;
+    if (strided) {
+        rw.first = lo + w * RPI; rw.step = nw * RPI; rw.sit = 1; rw.end = hi;
+        rw.ntiles = w < units ? (units - w + nw - 1) / nw : 0;
+    } else {
+        const int u0 = (int)(((long long)w * units) / nw), u1 = (int)(((long long)(w + 1) * units) / nw);
+        rw.first = lo + u0 * RPI; rw.step = RPI; rw.sit = 1; rw.ntiles = u1 - u0;
+        rw.end = lo + u1 * RPI < hi ? lo + u1 * RPI : hi;
+    }
+    return rw;
+}
+template <int RPI>
+__device__ __forceinline__ int walk_row(const RowWalk& rw, int k) { return rw.first + (k / RPI) * rw.step + (k % RPI) * rw.sit; }
+
+// QKV rows of one streaming wave; result = dot + bias as raw fp32.
 template <int NCH, bool EX>
-__device__ __forceinline__ void qkv_rows(const LayerParams& p, const half2_t (&x1)[NCH][4], int first, int stride, int lane,
+__device__ __forceinline__ void qkv_rows(const LayerParams& p, const half2_t (&x1)[NCH][4], const RowWalk& rw, int lane,
                                          RowTile<NCH, StageARpi<NCH>::value>& pre, RowPark& park) {
     constexpr int RPI = StageARpi<NCH>::value;
-    const int nq = 3 * p.H;
-    const int mine = first < nq ? (nq - first + stride - 1) / stride : 0;      // rows of this wave
+    const int first = rw.first, step = rw.step;
     gemv_tiles<NCH, RPI, EX>(
-        p.w_qkv, p.H, nq, stride, (mine + RPI - 1) / RPI, [=](int t) { return first + t * RPI * stride; }, x1, lane, pre, park,
+        p.w_qkv, p.H, rw.end, rw.sit, rw.ntiles, [=](int t) { return first + t * step; }, x1, lane, pre, park,
         [&](const RowPark& pk, int k0) {
             if (lane < pk.n) {
-                const int row = first + (k0 + lane) * stride;
+                const int row = walk_row<RPI>(rw, k0 + lane);
                 st_agent(p.qkv_raw + row, pk.slot[lane] + (float)p.b_qkv[row]);
             }
         });
 }
 template <int NCH, bool EX>
-__device__ __forceinline__ void qkv_prefetch(const LayerParams& p, int first, int stride, int lane,
+__device__ __forceinline__ void qkv_prefetch(const LayerParams& p, const RowWalk& rw, int lane,
                                              RowTile<NCH, StageARpi<NCH>::value>& pre) {
-    const int nq = 3 * p.H;
-    if (first < nq) load_row_tile<NCH, StageARpi<NCH>::value, EX>(pre, p.w_qkv, p.H, first, stride, nq, lane);
+    if (rw.ntiles > 0) load_row_tile<NCH, StageARpi<NCH>::value, EX>(pre, p.w_qkv, p.H, rw.first, rw.sit, rw.end, lane);
 }
 
-// MLP-up rows of one streaming wave: batches first, first+stride, ... of kUpRpi adjacent rows;
-// result = gelu(dot + bias) as fp16.
+// MLP-up rows of one streaming wave (tiles of kUpRpi adjacent rows); result = gelu(dot + bias) as fp16.
+// up_prefetch requests the first tile (before something slow: a LayerNorm, an event), up_rows consumes it.
 template <int NCH, bool EX>
-__device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], int first, int stride, int lane,
-                                        RowPark& park) {
-    const int nbatch = (p.F + kUpRpi - 1) / kUpRpi;
-    const int mine = first < nbatch ? (nbatch - first + stride - 1) / stride : 0;   // batches of this wave
-    if (mine == 0) return;
-    RowTile<NCH, kUpRpi> pre;
-    load_row_tile<NCH, kUpRpi, EX>(pre, p.w_up, p.H, first * kUpRpi, 1, p.F, lane);
+__device__ __forceinline__ void up_prefetch(const LayerParams& p, const RowWalk& rw, int lane, RowTile<NCH, kUpRpi>& pre) {
+    if (rw.ntiles > 0) load_row_tile<NCH, kUpRpi, EX>(pre, p.w_up, p.H, rw.first, rw.sit, rw.end, lane);
+}
+template <int NCH, bool EX>
+__device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], const RowWalk& rw, int lane,
+                                        RowTile<NCH, kUpRpi>& pre, RowPark& park) {
+    const int first = rw.first, step = rw.step;
     gemv_tiles<NCH, kUpRpi, EX>(
-        p.w_up, p.H, p.F, 1, mine, [=](int t) { return (first + t * stride) * kUpRpi; }, x2, lane, pre, park,
+        p.w_up, p.H, rw.end, rw.sit, rw.ntiles, [=](int t) { return first + t * step; }, x2, lane, pre, park,
         [&](const RowPark& pk, int k0) {
             if (lane < pk.n) {
-                const int k = k0 + lane;
-                const int row = (first + (k / kUpRpi) * stride) * kUpRpi + (k % kUpRpi);
+                const int row = walk_row<kUpRpi>(rw, k0 + lane);
                 st_agent(p.inter + row, (half_t)gelu_tanh(pk.slot[lane] + (float)p.b_up[row]));
             }
         });
@@ -74,16 +95,26 @@ __device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2
 template <int NCH, bool EX>
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_a(LayerParams p) {
     __shared__ float park_mem[kStreamers][kParkRows];
+    __shared__ LnShared<NCH> lns;
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int gw = blockIdx.x * kStreamers + wave, nw = gridDim.x * kStreamers;
     RowPark park{park_mem[wave], 0};
+    const bool strided = p.row_walk_strided != 0;
+    const RowWalk qw = row_walk<StageARpi<NCH>::value>(strided, gw, nw, 0, 3 * p.H);
+    LnOwn<NCH, kStreamers> own;
+    ln_coop_load<NCH, kStreamers, true>(own, p.x, p.H, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, wave, lane);
+    __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
     RowTile<NCH, StageARpi<NCH>::value> t0;
-    qkv_prefetch<NCH, EX>(p, gw, nw, lane, t0);
+    qkv_prefetch<NCH, EX>(p, qw, lane, t0);
+    ln_coop_finish<NCH, kStreamers, true>(own, p.H, p.eps, lns, wave, lane);
     half2_t xr[NCH][4];
-    const LnStats st = ln_first<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, lane, xr);
-    qkv_rows<NCH, EX>(p, xr, gw, nw, lane, t0, park);
-    ln_affine<NCH>(p.x, p.H, st, p.ln2_w, p.ln2_b, lane, xr);
-    up_rows<NCH, EX>(p, xr, gw, nw, lane, park);
+    ln_fetch<NCH>(lns, 0, lane, xr);
+    qkv_rows<NCH, EX>(p, xr, qw, lane, t0, park);
+    const RowWalk uw = row_walk<kUpRpi>(strided, gw, nw, 0, p.F);
+    RowTile<NCH, kUpRpi> u0;
+    up_prefetch<NCH, EX>(p, uw, lane, u0);
+    ln_fetch<NCH>(lns, 1, lane, xr);
+    up_rows<NCH, EX>(p, xr, uw, lane, u0, park);
 }
 
 // one (head, split) item per wave
@@ -100,14 +131,17 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
     __shared__ StageCShared sh;
     const int wave = first_lane(threadIdx.x >> 6);
     const StageC c = make_stage_c(p);
-    stage_c_rows<NCH, CPD>(c, blockIdx.x, gridDim.x, sh, true, wave, wave, kStreamers, [] {}, [] {});
+    stage_c_rows<NCH, CPD>(c, blockIdx.x, gridDim.x, sh, true, wave, wave, kStreamers, [](int) {}, [] {});
 }
 
 // ---- fused mode: one persistent launch ---------------------------------------------------------
 // One workgroup per compute unit, eight waves: four streaming waves (one per SIMD) and four helper waves.
 //   streaming wave: first QKV tile in flight -> LayerNorm -> its QKV rows -> bump kBarQkv -> its MLP-up
-//                   rows -> bump kBarUp -> (helps with attention items if any are left) -> MLP-down rows
-//                   of stage C (first weight tile in flight, then wait for kBarUp).
+//                   rows, phase by phase, bumping kBarUp + g after phase g -> (helps with attention items
+//                   if any are left) -> MLP-down rows of stage C, phase by phase (first weight tile in
+//                   flight, then wait for kBarUp + g): the first down phase only needs the first up phase
+//                   of every workgroup, so a workgroup that is late with its MLP-up rows holds up nobody
+//                   until the second half of the down pass.
 //   helper wave:    waits for kBarQkv, then takes (head, split) attention items from the workgroup's
 //                   queue at raised wave priority, then does the O-projection rows of stage C (first
 //                   rows in flight, then wait for kBarHeads).  Attention is a chain of dependent memory
@@ -116,7 +150,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
 //   all waves:      row reduction in LDS, bias, residual.
 // The last workgroup to leave zeroes the counters for the next launch.  All workgroups must be
 // co-resident (the host launches one per compute unit); every wait is bounded.
-struct FusedShared { int attn_next; int arrived[2]; };
+struct FusedShared { int attn_next; int arrived[1 + kUpPhases]; };
 
 __device__ __forceinline__ int lds_take(int* p) { return __hip_atomic_fetch_add(p, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 
@@ -124,16 +158,33 @@ template <int NCH, int CPD, bool EX>
 __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     __shared__ FusedShared q;
     __shared__ StageCShared shc;
+    __shared__ LnShared<NCH> lns;
     __shared__ float park_mem[kStreamers][kParkRows];
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int G = gridDim.x, b = blockIdx.x;
     const int nsw = G * kStreamers;                 // streaming waves in the grid
     int* status = p.bar + kBarStatus;
-    if (threadIdx.x == 0) { q.attn_next = 0; q.arrived[0] = 0; q.arrived[1] = 0; }
+    if (threadIdx.x <= kUpPhases) { q.attn_next = 0; q.arrived[threadIdx.x] = 0; }
     __syncthreads();
     trace_mark(p, 0);
     trace_value(p, 8, __builtin_amdgcn_s_getreg((3 << 11) | 20));   // XCC_ID: which XCD this workgroup runs on
     trace_value(p, 11, __builtin_amdgcn_s_getreg((31 << 11) | 4));  // HW_ID: wave slot, SIMD, CU, SE
+
+    // LayerNorm by all eight waves; the streaming waves request their first QKV tile behind the (few)
+    // LayerNorm loads, so the tile is on its way while the statistics are computed
+    constexpr int kFusedWaves = 2 * kStreamers;
+    const bool strided = p.row_walk_strided != 0;
+    const int sgw = b * kStreamers + wave;          // streaming waves only
+    const RowWalk qw = row_walk<StageARpi<NCH>::value>(strided, sgw, nsw, 0, 3 * p.H);
+    RowTile<NCH, StageARpi<NCH>::value> t0;
+    {
+        LnOwn<NCH, kFusedWaves> own;
+        ln_coop_load<NCH, kFusedWaves, true>(own, p.x, p.H, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, wave, lane);
+        __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
+        if (wave < kStreamers) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
+        ln_coop_finish<NCH, kFusedWaves, true>(own, p.H, p.eps, lns, wave, lane);
+    }
+    trace_mark(p, 1);
 
     const int S = load_seq_len(p);
     const int nsplit = effective_split(p, S);
@@ -153,20 +204,28 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     };
 
     if (wave < kStreamers) {
-        const int sgw = b * kStreamers + wave;
         RowPark park{park_mem[wave], 0};
         half2_t xr[NCH][4];   // ln1(x) for the QKV rows, then ln2(x) for the MLP-up rows
-        RowTile<NCH, StageARpi<NCH>::value> t0;
-        qkv_prefetch<NCH, EX>(p, sgw, nsw, lane, t0);
-        const LnStats st = ln_first<NCH>(p.x, p.H, p.eps, p.ln_w, p.ln_b, lane, xr);
-        trace_mark(p, 1);
-        qkv_rows<NCH, EX>(p, xr, sgw, nsw, lane, t0, park);
+        ln_fetch<NCH>(lns, 0, lane, xr);
+        qkv_rows<NCH, EX>(p, xr, qw, lane, t0, park);
         event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], kStreamers);
         trace_mark(p, 2);
-        ln_affine<NCH>(p.x, p.H, st, p.ln2_w, p.ln2_b, lane, xr);
-        up_rows<NCH, EX>(p, xr, sgw, nsw, lane, park);
-        event_arrive(p.bar, p.grp, p.mbox, kBarUp, G, &q.arrived[1], kStreamers);
-        trace_mark(p, 5);
+        ln_fetch<NCH>(lns, 1, lane, xr);
+        // MLP-up rows in kUpPhases ranges, an event after each; the first tile of the next range is
+        // requested before the event, so the wave is not left without loads in flight
+        RowTile<NCH, kUpRpi> u0;
+        RowWalk uw = row_walk<kUpRpi>(strided, sgw, nsw, 0, up_phase_rows(CPD, 0, p.F));
+        up_prefetch<NCH, EX>(p, uw, lane, u0);
+#pragma unroll
+        for (int g = 0; g < kUpPhases; ++g) {
+            up_rows<NCH, EX>(p, xr, uw, lane, u0, park);
+            if (g + 1 < kUpPhases) {
+                uw = row_walk<kUpRpi>(strided, sgw, nsw, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F));
+                up_prefetch<NCH, EX>(p, uw, lane, u0);
+            }
+            event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &q.arrived[1 + g], kStreamers);
+            trace_mark(p, g == kUpPhases - 1 ? 5 : 12);
+        }
         event_wait(p.mbox, kBarQkv, status);
         take_attention_items();
     } else {
@@ -181,7 +240,7 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
         const bool streamer = wave < kStreamers;
         stage_c_rows<NCH, CPD>(
             c, b, G, shc, streamer, wave, streamer ? -1 : wave - kStreamers, kStreamers,
-            [&] { event_wait(p.mbox, kBarUp, status); trace_mark(p, 6); },
+            [&](int g) { event_wait(p.mbox, kBarUp + g, status); trace_mark(p, g == 0 ? 6 : 13); },
             [&] { event_wait(p.mbox, kBarHeads, status); trace_mark(p, 7); });
     }
     trace_mark(p, 10);
@@ -225,18 +284,24 @@ __global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __res
     constexpr int RPIA = StageARpi<NCH>::value;
     __shared__ float park_mem[NWV][kParkRows];
     RowPark park{park_mem[wave], 0};
+    const RowWalk rw = row_walk<RPIA>(false, gw, nw, 0, vocab);   // contiguous rows per wave
+    __shared__ LnShared<NCH> lns;
+    LnOwn<NCH, NWV> own;
+    ln_coop_load<NCH, NWV, false>(own, x, H, ln_w, ln_b, nullptr, nullptr, wave, lane);
+    __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
     RowTile<NCH, RPIA> t0;
-    if (gw < vocab) load_row_tile<NCH, RPIA, EX>(t0, W, H, gw, nw, vocab, lane);
+    if (rw.ntiles > 0) load_row_tile<NCH, RPIA, EX>(t0, W, H, rw.first, rw.sit, rw.end, lane);
+    ln_coop_finish<NCH, NWV, false>(own, H, eps, lns, wave, lane);
     half2_t x1[NCH][4];
-    ln_first<NCH>(x, H, eps, ln_w, ln_b, lane, x1);
+    ln_fetch<NCH>(lns, 0, lane, x1);
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    const int mine = gw < vocab ? (vocab - gw + nw - 1) / nw : 0;
+    const int first = rw.first, step = rw.step;
     gemv_tiles<NCH, RPIA, EX>(
-        W, H, vocab, nw, (mine + RPIA - 1) / RPIA, [=](int t) { return gw + t * RPIA * nw; }, x1, lane, t0, park,
+        W, H, rw.end, rw.sit, rw.ntiles, [=](int t) { return first + t * step; }, x1, lane, t0, park,
         [&](const RowPark& pk, int k0) {
             if (lane < pk.n) {
-                const int row = gw + (k0 + lane) * nw;
+                const int row = walk_row<RPIA>(rw, k0 + lane);
                 const float v = pk.slot[lane];
                 logits[row] = v;
                 if (v > bv || (v == bv && row < bi)) { bv = v; bi = row; }
@@ -451,6 +516,13 @@ bool shape_supported(const Plan& pl) {
 
 // upper bound of the KV splits per head the kernels will use for a sequence length (device code
 // computes the same value from the actual length: effective_split)
+// workgroups of a streaming launch: one per compute unit
+int streaming_grid() {
+    DeviceInfo& di = device_info();
+    const int cus = di.cus > 0 ? di.cus : 256;
+    return cus * env_int("CFPP_WG_PER_CU", 1);
+}
+
 int split_bound(int seq_hint, int max_split) {
     int n = (seq_hint + kSplitRows - 1) / kSplitRows;
     n = n < 1 ? 1 : n;
@@ -498,6 +570,11 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     p.max_split = env_int("CFPP_MAX_SPLIT", kMaxSplit);
     if (p.max_split < 1) p.max_split = 1;
     if (p.max_split > kMaxSplit) p.max_split = kMaxSplit;
+    // one (head, split) item per attention wave of the fused launch at most: an item more than that would
+    // start only after some wave has finished its first one, and end the attention phase late
+    const int per_head = streaming_grid() * kStreamers / (d->heads > 0 ? d->heads : 1);
+    if (p.max_split > per_head) p.max_split = per_head < 1 ? 1 : per_head;
+    p.row_walk_strided = env_int("CFPP_ROW_WALK_STRIDED", 0);
     char* ws = reinterpret_cast<char*>(workspace);
     p.qkv_raw = reinterpret_cast<float*>(ws + L.qkv_raw);
     p.attn_vec = reinterpret_cast<half_t*>(ws + L.attn_vec);
@@ -518,11 +595,7 @@ int seq_hint_of(const cfpp_neox_io* io) {
     return io->d_seq_len ? (io->max_seq_len > 0 ? io->max_seq_len : io->cache_rows) : io->seq_len;
 }
 
-int grid_for_streaming(const Plan&) {
-    DeviceInfo& di = device_info();
-    const int cus = di.cus > 0 ? di.cus : 256;
-    return cus * env_int("CFPP_WG_PER_CU", 1);
-}
+int grid_for_streaming(const Plan&) { return streaming_grid(); }
 
 int run_split(const Plan& pl, LayerParams& p, int seq_hint, hipStream_t st) {
     const int grid = grid_for_streaming(pl);
