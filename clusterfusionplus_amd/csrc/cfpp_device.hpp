@@ -44,13 +44,16 @@ constexpr float kNegBig = -1.0e30f;
 constexpr int kSpinLimit = 1 << 20;    // bounded device-side waits (order of a second)
 
 enum : int { kStatusSpin = 1, kStatusSeq = 2 };
-// counters in LayerParams::bar (self-resetting: the last workgroup to leave zeroes them)
+// Slots of LayerParams::bar.  The event counters reset themselves (the arrival that completes a count
+// stores zero); flags are not reset at all: a launch raises a flag by writing its tag, the launch
+// generation read from kBarGen plus one, and the last workgroup to leave stores that tag back.
 enum BarSlot : int {
     kBarQkv = 0,      // streaming waves that have written their QKV rows
     kBarUp = 1,       // kBarUp + g: streaming waves that have written their MLP-up rows of phase g (kUpPhases slots)
     kBarHeads = 3,    // heads whose attention output is merged
     kBarExit = 4,     // workgroups that have finished
-    kBarStatus = 5    // failure flags (kStatusSpin, kStatusSeq); not reset by the kernels
+    kBarStatus = 5,   // failure flags (kStatusSpin, kStatusSeq); never reset by the kernels
+    kBarGen = 6       // launch generation
 };
 
 struct LayerParams {
@@ -226,9 +229,10 @@ __device__ __forceinline__ int* group_counter(int* grp, int event, int g) {
     return grp + (event * kEventGroups + g) * kMailboxInts;
 }
 // Called by a whole wave after its stores: drains them and counts the arrival; `per_wg` waves of every
-// workgroup arrive (1 if lds_ctr is null).  The wave that completes the event raises mailbox slot
-// `event` of all `nwg` workgroups.  Returns true in that wave.
-__device__ __forceinline__ bool event_arrive(int* bar, int* grp, int* mbox, int event, int nwg, int* lds_ctr, int per_wg) {
+// workgroup arrive (1 if lds_ctr is null).  The wave that completes a count zeroes it for the next launch;
+// the one that completes the event writes `tag` into mailbox slot `event` of all `nwg` workgroups and
+// returns true.
+__device__ __forceinline__ bool event_arrive(int* bar, int* grp, int* mbox, int event, int nwg, int* lds_ctr, int per_wg, int tag) {
     const int lane = threadIdx.x & 63;
     drain_memory_ops();
     int go = 1;
@@ -239,38 +243,34 @@ __device__ __forceinline__ bool event_arrive(int* bar, int* grp, int* mbox, int 
     if (!go) return false;
     const int g = blockIdx.x % kEventGroups;
     const int gsize = (nwg - g + kEventGroups - 1) / kEventGroups;
-    if (lane == 0) go = (__hip_atomic_fetch_add(group_counter(grp, event, g), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gsize - 1);
+    int* gc = group_counter(grp, event, g);
+    if (lane == 0) {
+        go = (__hip_atomic_fetch_add(gc, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gsize - 1);
+        if (go) __hip_atomic_store(gc, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     go = __builtin_amdgcn_readfirstlane(go);
     if (!go) return false;
     const int ngroups = nwg < kEventGroups ? nwg : kEventGroups;
-    if (lane == 0) go = (__hip_atomic_fetch_add(bar + event, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngroups - 1);
+    if (lane == 0) {
+        go = (__hip_atomic_fetch_add(bar + event, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngroups - 1);
+        if (go) __hip_atomic_store(bar + event, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     go = __builtin_amdgcn_readfirstlane(go);
     if (!go) return false;
     if (mbox != nullptr) {
         for (int w = lane; w < nwg; w += kWave)
-            __hip_atomic_store(mbox + w * kMailboxInts + event, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(mbox + w * kMailboxInts + event, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     return true;
-}
-// A flat count for events with few arrivals (one per attention head).
-__device__ __forceinline__ void event_arrive_flat(int* ctr, int target, int* mbox, int slot, int nwg) {
-    const int lane = threadIdx.x & 63;
-    drain_memory_ops();
-    int last = 0;
-    if (lane == 0) last = (__hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == target - 1);
-    if (__builtin_amdgcn_readfirstlane(last)) {
-        for (int w = lane; w < nwg; w += kWave)
-            __hip_atomic_store(mbox + w * kMailboxInts + slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
 }
 // One lane polls this workgroup's mailbox line, the wave leaves together.  Data published before the
 // arrivals must be read with ld_agent / ld_agent16.  A wait that expires raises a status flag and
 // falls through.
-__device__ __forceinline__ void event_wait(const int* mbox, int slot, int* status) {
+__device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, int* status) {
     if ((threadIdx.x & 63) == 0) {
         const int* f = mbox + blockIdx.x * kMailboxInts + slot;
         int spins = 0;
-        while (counter_peek(f) == 0) {
+        while (counter_peek(f) != tag) {
             __builtin_amdgcn_s_sleep(2);
             if (++spins > kSpinLimit) { raise_status(status, kStatusSpin); break; }
         }
@@ -531,12 +531,24 @@ struct StageARpi { static constexpr int value = (16 / NCH) > 0 ? (16 / NCH) : 1;
 // NeoX rotate-half RoPE on the first `rot` dims of a head vector held in raw fp32 scratch
 // (reference include/5090/pythia_2b8/kernel.cuh:395-421): d < rot/2 -> v[d] cos[d] - v[d+rot/2] sin[d];
 // rot/2 <= d < rot -> v[d] cos[d] + v[d-rot/2] sin[d]; d >= rot passes through.
-// A lane produces dims d0 .. d0+7.  Every load (own values, rotation partners, cos, sin) is issued
-// before the first use, so the whole vector costs one memory round trip; dims >= rot use cos = 1 and
-// sin = 0 on their own value.
-__device__ __forceinline__ void rope_load8(const float* __restrict__ v, int d0, int rot, const float* __restrict__ cs,
-                                           const float* __restrict__ sn, bool act, float (&out)[8]) {
-    float a[8], pr[8], c[8], sg[8];
+// A lane produces dims d0 .. d0+7.  rope_coeffs fetches cos and the signed sin of those dims (1 and 0 for
+// dims >= rot): they do not depend on the layer's own results, so they can be requested early.
+// rope_load8 requests the lane's own values and their rotation partners together (one memory round trip).
+struct RopeCoeffs { float c[8], sg[8]; };
+__device__ __forceinline__ void rope_coeffs(int d0, int rot, const float* __restrict__ cs, const float* __restrict__ sn,
+                                            bool act, RopeCoeffs& rc) {
+    const int hr = rot >> 1;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int d = d0 + j;
+        const bool rotd = act && d < rot;
+        rc.c[j] = rotd ? cs[d] : 1.f;
+        rc.sg[j] = rotd ? (d < hr ? -sn[d] : sn[d]) : 0.f;
+    }
+}
+__device__ __forceinline__ void rope_load8(const float* __restrict__ v, int d0, int rot, const RopeCoeffs& rc, bool act,
+                                           float (&out)[8]) {
+    float a[8], pr[8];
     const int hr = rot >> 1;
     if (act) {
         ld_agent2(v + d0, a[0], a[1]); ld_agent2(v + d0 + 2, a[2], a[3]);
@@ -544,55 +556,80 @@ __device__ __forceinline__ void rope_load8(const float* __restrict__ v, int d0, 
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int d = d0 + j;
-            const bool rotd = d < rot;
-            const int pd = rotd ? (d < hr ? d + hr : d - hr) : d;
+            const int pd = d < rot ? (d < hr ? d + hr : d - hr) : d;
             pr[j] = ld_agent(v + pd);
-            c[j] = rotd ? cs[d] : 1.f;
-            sg[j] = rotd ? (d < hr ? -sn[d] : sn[d]) : 0.f;
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) out[j] = a[j] * c[j] + pr[j] * sg[j];
+        for (int j = 0; j < 8; ++j) out[j] = d0 + j < rot ? a[j] * rc.c[j] + pr[j] * rc.sg[j] : a[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) out[j] = 0.f;
+    }
+}
+__device__ __forceinline__ void raw_load8(const float* __restrict__ v, int d0, bool act, float (&out)[8]) {
+    if (act) {
+        ld_agent2(v + d0, out[0], out[1]); ld_agent2(v + d0 + 2, out[2], out[3]);
+        ld_agent2(v + d0 + 4, out[4], out[5]); ld_agent2(v + d0 + 6, out[6], out[7]);
     } else {
 #pragma unroll
         for (int j = 0; j < 8; ++j) out[j] = 0.f;
     }
 }
 
-// The wave's four 16-lane groups take cache rows begin+g, begin+g+4, ...; lane `sub` of a group holds
-// dims 8 sub .. 8 sub + 7 of its row (lanes with 8 sub >= D contribute nothing).  T rows per group are in
-// flight (32 rows per wave).  An item is a chain of dependent memory round trips, so everything that can
-// be requested early is: the first K/V tile goes out before q is fetched.
-// nwg_to_signal > 0 (fused kernel): a completed head counts towards the kBarHeads event of that many workgroups.
-__device__ __forceinline__ void attention_item(const LayerParams& p, int head, int sp, int nsplit, int S, int lane,
-                                               int nwg_to_signal) {
+// One (head, split) item: the wave's four 16-lane groups take cache rows begin+g, begin+g+4, ...; lane
+// `sub` of a group holds dims 8 sub .. 8 sub + 7 of its row (lanes with 8 sub >= D contribute nothing).
+// A tile is kAttnT rows per group (32 rows per wave).  An item is a chain of dependent memory round
+// trips, so everything that does not depend on this layer's QKV rows is requested ahead of them by
+// attn_prefetch: the first two K/V tiles and the RoPE coefficients.  In the fused kernel that happens while
+// the attention waves would otherwise sit waiting for the QKV rows.
+constexpr int kAttnT = 8;
+constexpr int kAttnTileRows = 4 * kAttnT;
+struct KvTile { u32x4 k[kAttnT], v[kAttnT]; };
+struct AttnItem {
+    int head, sp, nsplit, S, begin, end, ntiles;
+    KvTile t0, t1;
+    RopeCoeffs rc;
+};
+// tile i of the item; rows past the end re-read the last row (masked when used): no conditional loads
+__device__ __forceinline__ void attn_load_tile(const LayerParams& p, const AttnItem& it, KvTile& kv, int i, int lane) {
     const int grp = lane >> 4, sub = lane & 15;
-    const int D = p.D, H = p.H;
-    const bool act = sub * 8 < D;
-    const int d0 = act ? sub * 8 : 0;      // idle lanes read (and ignore) the first dims
-    const float* __restrict__ raw = p.qkv_raw + (size_t)head * 3 * D;
+    const int d0 = sub * 8 < p.D ? sub * 8 : 0;      // idle lanes read (and ignore) the first dims
+    const half_t* __restrict__ kc = p.k_cache + (size_t)it.head * p.D + d0;
+    const half_t* __restrict__ vc = p.v_cache + (size_t)it.head * p.D + d0;
+    const int r = it.begin + i * kAttnTileRows + grp;
+#pragma unroll
+    for (int t = 0; t < kAttnT; ++t) {
+        const int row = (r + t * 4 < it.end) ? r + t * 4 : it.end - 1;
+        kv.k[t] = ld16(kc + (size_t)row * p.H);
+        kv.v[t] = ld16(vc + (size_t)row * p.H);
+    }
+}
+__device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it, int head, int sp, int nsplit, int S, int lane) {
+    it.head = head; it.sp = sp; it.nsplit = nsplit; it.S = S;
+    const int chunk = (S + nsplit - 1) / nsplit;
+    it.begin = sp * chunk;
+    it.end = (it.begin + chunk < S) ? it.begin + chunk : S;
+    it.ntiles = it.begin < it.end ? (it.end - it.begin + kAttnTileRows - 1) / kAttnTileRows : 0;
+    if (it.ntiles > 0) attn_load_tile(p, it, it.t0, 0, lane);
+    if (it.ntiles > 1) attn_load_tile(p, it, it.t1, 1, lane);
+    const int sub = lane & 15;
+    const bool act = sub * 8 < p.D;
     const float* __restrict__ cs = p.cos + (size_t)S * p.rope_stride;   // stride 0: the row is the position
     const float* __restrict__ sn = p.sin + (size_t)S * p.rope_stride;
+    rope_coeffs(act ? sub * 8 : 0, p.rot, cs, sn, act, it.rc);
+}
 
-    const int chunk = (S + nsplit - 1) / nsplit;
-    const int begin = sp * chunk;
-    const int end = (begin + chunk < S) ? begin + chunk : S;
-    const half_t* __restrict__ kc = p.k_cache + (size_t)head * D + d0;
-    const half_t* __restrict__ vc = p.v_cache + (size_t)head * D + d0;
-    constexpr int T = 8;
-    u32x4 kk[T], vv[T];
-    // rows past the end re-read the last row (masked below): no conditional loads
-    auto load_kv = [&](int r) {
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-            const int row = (r + t * 4 < end) ? r + t * 4 : end - 1;
-            kk[t] = ld16(kc + (size_t)row * H);
-            vv[t] = ld16(vc + (size_t)row * H);
-        }
-    };
-    if (begin < end) load_kv(begin + grp);
+// nwg_to_signal > 0 (fused kernel): a completed head counts towards the kBarHeads event of that many workgroups.
+__device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& it, int lane, int nwg_to_signal, int tag) {
+    const int grp = lane >> 4, sub = lane & 15;
+    const int D = p.D, H = p.H;
+    const int head = it.head, sp = it.sp, nsplit = it.nsplit, S = it.S, end = it.end;
+    const bool act = sub * 8 < D;
+    const int d0 = act ? sub * 8 : 0;
+    const float* __restrict__ raw = p.qkv_raw + (size_t)head * 3 * D;
 
     float q[8];
-    rope_load8(raw, d0, p.rot, cs, sn, act, q);
+    rope_load8(raw, d0, p.rot, it.rc, act, q);
 #pragma unroll
     for (int j = 0; j < 8; ++j) q[j] *= p.qscale;
 
@@ -603,8 +640,8 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
     // the new token: split 0 owns it (appends it, returns it, and seeds its softmax state with it)
     if (sp == 0 && grp == 0) {
         float kf[8], vf[8];
-        rope_load8(raw + D, d0, p.rot, cs, sn, act, kf);
-        rope_load8(raw + 2 * D, d0, 0, cs, sn, act, vf);
+        rope_load8(raw + D, d0, p.rot, it.rc, act, kf);
+        raw_load8(raw + 2 * D, d0, act, vf);
         const u32x4 kp = pack8(kf), vp = pack8(vf);
         unpack8(kp, kf); unpack8(vp, vf);      // attend over the fp16 values the cache will hold
         if (act) {
@@ -625,13 +662,13 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
         for (int j = 0; j < 8; ++j) acc[j] = vf[j];
     }
 
-    for (int r = begin + grp; r - grp < end; r += 4 * T) {
-        if (r - grp != begin) load_kv(r);
-        float s[T], mt = m;
+    auto process = [&](const KvTile& kv, int i) {
+        const int r = it.begin + i * kAttnTileRows + grp;
+        float s[kAttnT], mt = m;
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
+        for (int t = 0; t < kAttnT; ++t) {
             float kf[8];
-            unpack8(kk[t], kf);
+            unpack8(kv.k[t], kf);
             float d = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) d += q[j] * kf[j];
@@ -644,15 +681,25 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[j] *= alpha;
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
+        for (int t = 0; t < kAttnT; ++t) {
             const float pt = (r + t * 4 < end) ? fast_exp2(s[t] - mt) : 0.f;
             float vf[8];
-            unpack8(vv[t], vf);
+            unpack8(kv.v[t], vf);
             l += pt;
 #pragma unroll
             for (int j = 0; j < 8; ++j) acc[j] += pt * vf[j];
         }
         m = mt;
+    };
+    if (it.ntiles > 0) process(it.t0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (it.ntiles > 2) attn_load_tile(p, it, it.t0, 2, lane);     // the third tile travels while the second is reduced
+    __builtin_amdgcn_sched_barrier(0);
+    if (it.ntiles > 1) process(it.t1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int i = 2; i < it.ntiles; ++i) {
+        if (i != 2) attn_load_tile(p, it, it.t0, i, lane);
+        process(it.t0, i);
     }
 
     // merge the four groups (lanes sub, sub+16, sub+32, sub+48 hold the same dims)
@@ -691,6 +738,18 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
         const size_t hb = (size_t)head * kMaxSplit;
         float mi = kNegBig, li = 0.f;
         if (lane < nsplit) ld_agent2(p.part_ml + (hb + lane) * 2, mi, li);
+        const int t2 = lane * 2;
+        const bool dact = t2 < D;
+        constexpr int kMergeBatch = 32;            // splits per memory round trip
+        float a0[kMergeBatch], a1[kMergeBatch];
+        auto load_acc = [&](int i0) {
+#pragma unroll
+            for (int u = 0; u < kMergeBatch; ++u) {
+                const int i = i0 + u < nsplit ? i0 + u : nsplit - 1;
+                ld_agent2(p.part_acc + (hb + i) * D + (dact ? t2 : 0), a0[u], a1[u]);
+            }
+        };
+        load_acc(0);     // requested together with the scales: one round trip for up to kMergeBatch splits
         float M = fmaxf(mi, xor_shfl(mi, 32));
         M = fmaxf(M, xor_shfl(M, 16));
         M = fmaxf(M, xor_shfl(M, 8));
@@ -699,18 +758,11 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
         M = fmaxf(M, xor_shfl(M, 1));
         const float sci = fast_exp2(mi - M);      // scale of split `lane`
         const float lsi = li * sci;
-        const int t2 = lane * 2;
-        const bool dact = t2 < D;
         float L = 0.f, A0 = 0.f, A1 = 0.f;
-        for (int i0 = 0; i0 < nsplit; i0 += 16) {     // 16 splits per memory round trip
-            float a0[16], a1[16];
+        for (int i0 = 0; i0 < nsplit; i0 += kMergeBatch) {
+            if (i0 != 0) load_acc(i0);
 #pragma unroll
-            for (int u = 0; u < 16; ++u) {
-                const int i = i0 + u < nsplit ? i0 + u : nsplit - 1;
-                ld_agent2(p.part_acc + (hb + i) * D + (dact ? t2 : 0), a0[u], a1[u]);
-            }
-#pragma unroll
-            for (int u = 0; u < 16; ++u) {
+            for (int u = 0; u < kMergeBatch; ++u) {
                 const bool in = i0 + u < nsplit;
                 const int i = in ? i0 + u : 0;
                 const float sc = in ? rl(sci, i) : 0.f;
@@ -724,7 +776,19 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, int head, i
             st_agent(reinterpret_cast<uint32_t*>(p.attn_vec + (size_t)head * D + t2), as_u32(o));
         }
         if (lane == 0) __hip_atomic_store(p.head_cnt + head, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (nwg_to_signal > 0) event_arrive_flat(p.bar + kBarHeads, p.heads, p.mbox, kBarHeads, nwg_to_signal);
+        if (nwg_to_signal > 0) {
+            // count the head; the wave that completes the count tells every workgroup
+            drain_memory_ops();
+            int all = 0;
+            if (lane == 0) {
+                all = (__hip_atomic_fetch_add(p.bar + kBarHeads, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.heads - 1);
+                if (all) __hip_atomic_store(p.bar + kBarHeads, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (first_lane(all)) {
+                for (int w = lane; w < nwg_to_signal; w += kWave)
+                    __hip_atomic_store(p.mbox + w * kMailboxInts + kBarHeads, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
     }
 }
 
@@ -878,6 +942,9 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
             }
         }
         if (o_index >= 0 && c.K1 > 0) {
+            // up to kORows rows of this wave are requested before the attention vector is waited for, so that
+            // only one more round trip (the vector itself) follows the wait
+            constexpr int kORows = 4;
             auto load_row = [&](u32x4 (&w)[NCH], int r) {
                 const int rr = r < b1 ? r : b1 - 1;
                 const half_t* rp = c.W1 + (size_t)rr * (size_t)c.K1;
@@ -887,8 +954,9 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
                     w[i] = ld_stream16(rp + (col < c.K1 ? col : 0));
                 }
             };
-            u32x4 wa[NCH], wb[NCH];
-            load_row(wa, b0 + o_index);
+            u32x4 w[kORows][NCH];
+#pragma unroll
+            for (int j = 0; j < kORows; ++j) load_row(w[j], b0 + o_index + j * n_o);
             if (first) o_ready();
             half2_t xs[NCH][4];
 #pragma unroll
@@ -898,28 +966,20 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
                 if (col < c.K1) xv = ld_agent16(c.x1 + col);
                 xs[i][0] = as_h2(xv.x); xs[i][1] = as_h2(xv.y); xs[i][2] = as_h2(xv.z); xs[i][3] = as_h2(xv.w);
             }
-            auto finish_row = [&](const u32x4 (&w)[NCH], int r) {
-                float acc = 0.f;
+            for (int r = b0 + o_index; r < b1; r += kORows * n_o) {
 #pragma unroll
-                for (int i = 0; i < NCH; ++i) acc = dot8(w[i], xs[i], acc);
-                acc = wave_sum(acc);
-                if (r < b1 && lane == 0) sh.red_o[r - b0] = acc;
-            };
-            int r = b0 + o_index;
-            for (; r + 2 * n_o < b1; r += 2 * n_o) {
-                load_row(wb, r + n_o);
-                finish_row(wa, r);
-                __builtin_amdgcn_sched_barrier(0);
-                load_row(wa, r + 2 * n_o);
-                finish_row(wb, r + n_o);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (r + n_o < b1) {
-                load_row(wb, r + n_o);
-                finish_row(wa, r);
-                finish_row(wb, r + n_o);
-            } else if (r < b1) {
-                finish_row(wa, r);
+                for (int j = 0; j < kORows; ++j) {
+                    float acc = 0.f;
+#pragma unroll
+                    for (int i = 0; i < NCH; ++i) acc = dot8(w[j][i], xs[i], acc);
+                    acc = wave_sum(acc);
+                    const int rj = r + j * n_o;
+                    if (rj < b1 && lane == 0) sh.red_o[rj - b0] = acc;
+                }
+                if (r + kORows * n_o < b1) {
+#pragma unroll
+                    for (int j = 0; j < kORows; ++j) load_row(w[j], r + (kORows + j) * n_o);
+                }
             }
         }
         first = false;

@@ -123,7 +123,11 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_b(LayerParams p) {
     const int S = load_seq_len(p);
     const int nsplit = effective_split(p, S);
     const int item = blockIdx.x * kStreamers + wave;
-    if (item < p.heads * nsplit) attention_item(p, item / nsplit, item % nsplit, nsplit, S, lane, 0);
+    if (item < p.heads * nsplit) {
+        AttnItem it;
+        attn_prefetch(p, it, item / nsplit, item % nsplit, nsplit, S, lane);
+        attention_item(p, it, lane, 0, 0);
+    }
 }
 
 template <int NCH, int CPD>
@@ -148,11 +152,10 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
 //                   round trips; it and the O projection run beside the MLP-up / MLP-down streaming
 //                   instead of in front of it.
 //   all waves:      row reduction in LDS, bias, residual.
-// The last workgroup to leave zeroes the counters for the next launch.  All workgroups must be
+// Nothing is reset at the end: counters zero themselves and flags carry a launch generation.  All workgroups must be
 // co-resident (the host launches one per compute unit); every wait is bounded.
-struct FusedShared { int attn_next; int arrived[1 + kUpPhases]; };
+struct FusedShared { int arrived[1 + kUpPhases]; };
 
-__device__ __forceinline__ int lds_take(int* p) { return __hip_atomic_fetch_add(p, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 
 template <int NCH, int CPD, bool EX>
 __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
@@ -164,8 +167,10 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     const int G = gridDim.x, b = blockIdx.x;
     const int nsw = G * kStreamers;                 // streaming waves in the grid
     int* status = p.bar + kBarStatus;
-    if (threadIdx.x <= kUpPhases) { q.attn_next = 0; q.arrived[threadIdx.x] = 0; }
+    if (threadIdx.x <= kUpPhases) q.arrived[threadIdx.x] = 0;
     __syncthreads();
+    // this launch's flag value: requested first, needed at the first event
+    const int gen = counter_peek(p.bar + kBarGen);
     trace_mark(p, 0);
     trace_value(p, 8, __builtin_amdgcn_s_getreg((3 << 11) | 20));   // XCC_ID: which XCD this workgroup runs on
     trace_value(p, 11, __builtin_amdgcn_s_getreg((31 << 11) | 4));  // HW_ID: wave slot, SIMD, CU, SE
@@ -185,30 +190,18 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
         ln_coop_finish<NCH, kFusedWaves, true>(own, p.H, p.eps, lns, wave, lane);
     }
     trace_mark(p, 1);
+    const int tag = first_lane(gen) + 1;
 
     const int S = load_seq_len(p);
     const int nsplit = effective_split(p, S);
     const int nitems = p.heads * nsplit;
     const int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
-    auto take_attention_items = [&] {
-        for (;;) {
-            int t = 0;
-            if (lane == 0) t = lds_take(&q.attn_next);
-            t = first_lane(t);
-            if (t >= attn_count) break;
-            const int item = b + t * G;
-            trace_mark(p, 3);
-            attention_item(p, item / nsplit, item % nsplit, nsplit, S, lane, G);
-            trace_mark(p, 4);
-        }
-    };
-
     if (wave < kStreamers) {
         RowPark park{park_mem[wave], 0};
         half2_t xr[NCH][4];   // ln1(x) for the QKV rows, then ln2(x) for the MLP-up rows
         ln_fetch<NCH>(lns, 0, lane, xr);
         qkv_rows<NCH, EX>(p, xr, qw, lane, t0, park);
-        event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], kStreamers);
+        event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], kStreamers, tag);
         trace_mark(p, 2);
         ln_fetch<NCH>(lns, 1, lane, xr);
         // MLP-up rows in kUpPhases ranges, an event after each; the first tile of the next range is
@@ -223,15 +216,23 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
                 uw = row_walk<kUpRpi>(strided, sgw, nsw, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F));
                 up_prefetch<NCH, EX>(p, uw, lane, u0);
             }
-            event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &q.arrived[1 + g], kStreamers);
+            event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &q.arrived[1 + g], kStreamers, tag);
             trace_mark(p, g == kUpPhases - 1 ? 5 : 12);
         }
-        event_wait(p.mbox, kBarQkv, status);
-        take_attention_items();
     } else {
-        event_wait(p.mbox, kBarQkv, status);
-        __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
-        take_attention_items();
+        // attention wave hw takes the (head, split) items b + (hw + 4 k) G; what does not depend on the QKV
+        // rows (first K/V tiles, RoPE coefficients) is requested before waiting for them
+        const int hw = wave - kStreamers;
+        // (the host caps the KV splits so that no wave has more than one item: attn_count <= kStreamers)
+        if (hw < attn_count) {
+            AttnItem it;
+            attn_prefetch(p, it, (b + hw * G) / nsplit, (b + hw * G) % nsplit, nsplit, S, lane);
+            event_wait(p.mbox, kBarQkv, tag, status);
+            __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
+            trace_mark(p, 3);
+            attention_item(p, it, lane, G, tag);
+            trace_mark(p, 4);
+        }
         __builtin_amdgcn_s_setprio(0);
     }
     trace_mark(p, 9);
@@ -240,23 +241,14 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
         const bool streamer = wave < kStreamers;
         stage_c_rows<NCH, CPD>(
             c, b, G, shc, streamer, wave, streamer ? -1 : wave - kStreamers, kStreamers,
-            [&](int g) { event_wait(p.mbox, kBarUp + g, status); trace_mark(p, g == 0 ? 6 : 13); },
-            [&] { event_wait(p.mbox, kBarHeads, status); trace_mark(p, 7); });
+            [&](int g) { event_wait(p.mbox, kBarUp + g, tag, status); trace_mark(p, g == 0 ? 6 : 13); },
+            [&] { event_wait(p.mbox, kBarHeads, tag, status); trace_mark(p, 7); });
     }
     trace_mark(p, 10);
-    // the last workgroup to leave re-arms the counters and mailboxes for the next launch
-    __shared__ int last_out;
+    // the last workgroup to leave publishes the new generation: flags of this launch turn stale
     if (wave == 0) {
-        const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1);
-        if (lane == 0) last_out = last;
-    }
-    __syncthreads();
-    if (last_out) {
-        for (int i = threadIdx.x; i < G * kMailboxInts; i += blockDim.x)
-            __hip_atomic_store(p.mbox + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (int i = threadIdx.x; i < (kBarExit + 1) * kEventGroups * kMailboxInts; i += blockDim.x)
-            __hip_atomic_store(p.grp + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (threadIdx.x <= kBarExit) __hip_atomic_store(p.bar + threadIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1, tag);
+        if (last && lane == 0) __hip_atomic_store(p.bar + kBarGen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -523,6 +515,13 @@ int streaming_grid() {
     return cus * env_int("CFPP_WG_PER_CU", 1);
 }
 
+// workgroups of the fused launch: one per compute unit, all co-resident
+int fused_grid() {
+    DeviceInfo& di = device_info();
+    const int grid = di.cus > 0 ? di.cus : 256;
+    return grid > kMaxGrid ? kMaxGrid : grid;
+}
+
 int split_bound(int seq_hint, int max_split) {
     int n = (seq_hint + kSplitRows - 1) / kSplitRows;
     n = n < 1 ? 1 : n;
@@ -572,7 +571,7 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     if (p.max_split > kMaxSplit) p.max_split = kMaxSplit;
     // one (head, split) item per attention wave of the fused launch at most: an item more than that would
     // start only after some wave has finished its first one, and end the attention phase late
-    const int per_head = streaming_grid() * kStreamers / (d->heads > 0 ? d->heads : 1);
+    const int per_head = fused_grid() * kStreamers / (d->heads > 0 ? d->heads : 1);
     if (p.max_split > per_head) p.max_split = per_head < 1 ? 1 : per_head;
     p.row_walk_strided = env_int("CFPP_ROW_WALK_STRIDED", 0);
     char* ws = reinterpret_cast<char*>(workspace);
@@ -647,9 +646,9 @@ int cfpp_neox_layer_decode(const cfpp_neox_dims* dims, const cfpp_neox_weights* 
     if (rc) return rc;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (mode == CFPP_MODE_SPLIT) return run_split(pl, p, seq_hint_of(io), st);
-    DeviceInfo& di = device_info();
-    int grid = di.cus > 0 ? di.cus : 256;
-    if (grid > kMaxGrid) grid = kMaxGrid;
+    const int grid = fused_grid();
+    // the fused kernel gives every attention wave at most one (head, split) item
+    if (p.heads > grid * kStreamers) return run_split(pl, p, seq_hint_of(io), st);
     return launch_fused(pl, p, grid, st);
 }
 
