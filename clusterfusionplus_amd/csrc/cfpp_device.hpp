@@ -69,6 +69,7 @@ struct LayerParams {
     const int* d_seq_len;
     int max_split;      // cap on the KV splits per head (<= kMaxSplit)
     int row_walk_strided;   // streaming waves take interleaved instead of contiguous row ranges
+    int dyn_up;             // MLP-up tiles handed out dynamically within teams of workgroups: 1 yes, 0 no, -1 by size
     // scratch
     float* qkv_raw;     // [3H] fp32: W_qkv ln1(x) + b_qkv, before RoPE
     half_t* attn_vec;   // [H] fp16: merged attention output (input of the O projection)
@@ -79,6 +80,7 @@ struct LayerParams {
     int* bar;           // device-wide counters, see BarSlot
     int* grp;           // [events][kEventGroups] group counters, one 64-byte line each
     int* mbox;          // [kMaxGrid][kMailboxInts] event flags, one line per workgroup
+    int* team;          // [1 + kUpPhases][kMaxGrid / kTeamWgs][kMailboxInts] ticket counters of the tile teams (QKV, MLP-up phases)
     // stage-C selection (split API halves)
     const half_t* c_base0;   // residual terms added to the output (nullable)
     const half_t* c_base1;
@@ -518,6 +520,124 @@ __device__ __forceinline__ void gemv_tiles(const half_t* __restrict__ W, int K, 
         __builtin_amdgcn_sched_barrier(0);
         flush(park, done);
         done += park.n;
+        park.n = 0;
+    }
+}
+
+// ---- dynamically shared tiles ---------------------------------------------------------------------
+// Compute units do not stream at the same speed (whole chiplets differ by tens of percent, differently
+// from machine to machine), so equal static shares leave the fast ones waiting for the slowest.  A team
+// of `nw` waves (the streaming waves of kTeamWgs consecutive workgroups, which the dispatcher places on
+// different chiplets) therefore shares the `ntiles` tiles of a row range: wave j starts with tiles j and
+// j + nw, and every further tile is a ticket from the team's counter, requested two tiles ahead of its use
+// (the atomic is issued before the loads of the tile in between, so its result is back before theirs).
+// Every wave ends with exactly one ticket past the end, so a team issues max(ntiles - 2 nw, 0) + nw
+// requests per pass; the wave that gets the last of them zeroes the counter for the next launch.
+constexpr int kTeamWgs = 8;
+struct TileTeam {
+    int* counter;      // the team's ticket counter (own 64-byte line), zero between launches
+    int j, nw;         // this wave's index in the team, waves in the team
+    int row0;          // first row of the team's range
+    int ntiles;        // tiles (of RPI adjacent rows) in the range
+    int end;           // rows >= end do not exist
+};
+struct RowParkIds {
+    float* slot;       // this wave's kParkRows floats in LDS
+    int* row;          // and the rows they belong to (-1: none)
+    int n;
+};
+__device__ __forceinline__ int ticket_request(int* counter, int lane) {
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return old;     // meaningful in lane 0; read with first_lane() when needed
+}
+template <int NCH, int RPI>
+__device__ __forceinline__ void finish_team_tile(const RowTile<NCH, RPI>& t, const half2_t (&x)[NCH][4], int row, int end, int lane,
+                                                 RowParkIds& park) {
+#pragma unroll
+    for (int j = 0; j < RPI; ++j) {
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) acc = dot8(t.w[j][i], x[i], acc);
+        acc = wave_sum(acc);
+        if (lane == 0) {
+            park.slot[park.n + j] = acc;
+            park.row[park.n + j] = row + j < end ? row + j : -1;
+        }
+    }
+    park.n += RPI;
+}
+// team_prefetch requests the wave's first ticket and its two static tiles (before something slow: the
+// LayerNorm, an event); gemv_team consumes them.  flush(park) runs outside the streaming loop, when the
+// park is full and at the end; parked value k belongs to row park.row[k].
+template <int NCH, int RPI>
+struct TeamTiles {
+    RowTile<NCH, RPI> a, b;
+    int req;
+};
+template <int NCH, int RPI, bool EXACT>
+__device__ __forceinline__ void team_prefetch(const half_t* __restrict__ W, int K, const TileTeam& tm, int lane,
+                                              TeamTiles<NCH, RPI>& tt) {
+    tt.req = ticket_request(tm.counter, lane);
+    if (tm.j < tm.ntiles) load_row_tile<NCH, RPI, EXACT>(tt.a, W, K, tm.row0 + tm.j * RPI, 1, tm.end, lane);
+}
+template <int NCH, int RPI, bool EXACT, class Flush>
+__device__ __forceinline__ void gemv_team(const half_t* __restrict__ W, int K, const TileTeam& tm, const half2_t (&x)[NCH][4],
+                                          int lane, TeamTiles<NCH, RPI>& tt, RowParkIds& park, Flush&& flush) {
+    static_assert(kParkRows >= 3 * RPI, "tile larger than the park");
+    const int total = (tm.ntiles > 2 * tm.nw ? tm.ntiles - 2 * tm.nw : 0) + tm.nw;    // requests per pass
+    auto row_of = [&](int t) { return tm.row0 + t * RPI; };
+    auto load = [&](RowTile<NCH, RPI>& t, int i) { load_row_tile<NCH, RPI, EXACT>(t, W, K, row_of(i), 1, tm.end, lane); };
+    auto retire = [&](int old) {      // the team's last request re-arms the counter
+        if (lane == 0 && old == total - 1) __hip_atomic_store(tm.counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    int req = tt.req;
+    int tA = tm.j, tB = tm.j + tm.nw;
+    if (tA >= tm.ntiles) {            // nothing for this wave: its one request is past the end
+        retire(req);
+        return;
+    }
+    if (tB >= tm.ntiles) {            // one tile only
+        finish_team_tile<NCH, RPI>(tt.a, x, row_of(tA), tm.end, lane, park);
+        retire(req);
+        flush(park);
+        park.n = 0;
+        return;
+    }
+    load(tt.b, tB);
+    bool more = true;
+    while (more) {
+        // the streaming loop: no stores, no conditional loads; it is left when the tickets run out or the
+        // park is full
+        while (park.n + 3 * RPI <= kParkRows) {     // a trip parks up to three tiles
+            finish_team_tile<NCH, RPI>(tt.a, x, row_of(tA), tm.end, lane, park);
+            int old = first_lane(req);
+            int tn = 2 * tm.nw + old;
+            if (tn >= tm.ntiles) {
+                retire(old);
+                finish_team_tile<NCH, RPI>(tt.b, x, row_of(tB), tm.end, lane, park);
+                more = false;
+                break;
+            }
+            req = ticket_request(tm.counter, lane);
+            load(tt.a, tn);
+            tA = tn;
+            __builtin_amdgcn_sched_barrier(0);
+            finish_team_tile<NCH, RPI>(tt.b, x, row_of(tB), tm.end, lane, park);
+            old = first_lane(req);
+            tn = 2 * tm.nw + old;
+            if (tn >= tm.ntiles) {
+                retire(old);
+                finish_team_tile<NCH, RPI>(tt.a, x, row_of(tA), tm.end, lane, park);
+                more = false;
+                break;
+            }
+            req = ticket_request(tm.counter, lane);
+            load(tt.b, tn);
+            tB = tn;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        flush(park);
         park.n = 0;
     }
 }

@@ -89,6 +89,46 @@ __device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2
         });
 }
 
+// The rows [lo, hi) of one pass (0: QKV, 1 + g: MLP-up phase g), as tiles of RPI rows shared dynamically
+// by the streaming waves of this workgroup's team.
+template <int RPI>
+__device__ __forceinline__ TileTeam make_team(const LayerParams& p, int pass, int lo, int hi, int b, int G, int wave) {
+    const int nteams = (G + kTeamWgs - 1) / kTeamWgs, k = b / kTeamWgs;
+    const int wgs = (G - k * kTeamWgs) < kTeamWgs ? (G - k * kTeamWgs) : kTeamWgs;
+    const int T = (hi - lo + RPI - 1) / RPI;
+    const int t0 = (int)(((long long)T * k) / nteams), t1 = (int)(((long long)T * (k + 1)) / nteams);
+    TileTeam tm;
+    tm.counter = p.team + ((size_t)pass * (kMaxGrid / kTeamWgs) + k) * kMailboxInts;
+    tm.j = (b - k * kTeamWgs) * kStreamers + wave;
+    tm.nw = wgs * kStreamers;
+    tm.row0 = lo + t0 * RPI;
+    tm.ntiles = t1 - t0;
+    tm.end = hi;
+    return tm;
+}
+// QKV rows: result = dot + bias as raw fp32
+template <int NCH, bool EX>
+__device__ __forceinline__ void qkv_team_rows(const LayerParams& p, const half2_t (&x1)[NCH][4], const TileTeam& tm, int lane,
+                                              TeamTiles<NCH, StageARpi<NCH>::value>& tt, RowParkIds& park) {
+    gemv_team<NCH, StageARpi<NCH>::value, EX>(p.w_qkv, p.H, tm, x1, lane, tt, park, [&](const RowParkIds& pk) {
+        if (lane < pk.n) {
+            const int row = pk.row[lane];
+            if (row >= 0) st_agent(p.qkv_raw + row, pk.slot[lane] + (float)p.b_qkv[row]);
+        }
+    });
+}
+// MLP-up rows: result = gelu(dot + bias) as fp16
+template <int NCH, bool EX>
+__device__ __forceinline__ void up_team_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], const TileTeam& tm, int lane,
+                                             TeamTiles<NCH, kUpRpi>& tt, RowParkIds& park) {
+    gemv_team<NCH, kUpRpi, EX>(p.w_up, p.H, tm, x2, lane, tt, park, [&](const RowParkIds& pk) {
+        if (lane < pk.n) {
+            const int row = pk.row[lane];
+            if (row >= 0) st_agent(p.inter + row, (half_t)gelu_tanh(pk.slot[lane] + (float)p.b_up[row]));
+        }
+    });
+}
+
 // ---- split mode: one launch per stage ----------------------------------------------------------
 // Four waves per workgroup everywhere: one per SIMD.  A second wave on a SIMD gets far less of the
 // memory pipeline than the first while both stream, so extra streaming waves only add imbalance.
@@ -163,6 +203,7 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     __shared__ StageCShared shc;
     __shared__ LnShared<NCH> lns;
     __shared__ float park_mem[kStreamers][kParkRows];
+    __shared__ int park_rows[kStreamers][kParkRows];
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int G = gridDim.x, b = blockIdx.x;
     const int nsw = G * kStreamers;                 // streaming waves in the grid
@@ -178,10 +219,9 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     // LayerNorm by all eight waves; the streaming waves request their first QKV tile behind the (few)
     // LayerNorm loads, so the tile is on its way while the statistics are computed
     constexpr int kFusedWaves = 2 * kStreamers;
-    const bool strided = p.row_walk_strided != 0;
-    const int sgw = b * kStreamers + wave;          // streaming waves only
-    const RowWalk qw = row_walk<StageARpi<NCH>::value>(strided, sgw, nsw, 0, 3 * p.H);
-    RowTile<NCH, StageARpi<NCH>::value> t0;
+    constexpr int RPIA = StageARpi<NCH>::value;
+    const RowWalk qw = row_walk<RPIA>(false, b * kStreamers + wave, nsw, 0, 3 * p.H);     // streaming waves only
+    RowTile<NCH, RPIA> t0;
     {
         LnOwn<NCH, kFusedWaves> own;
         ln_coop_load<NCH, kFusedWaves, true>(own, p.x, p.H, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, wave, lane);
@@ -197,27 +237,50 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     const int nitems = p.heads * nsplit;
     const int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
     if (wave < kStreamers) {
-        RowPark park{park_mem[wave], 0};
+        RowPark spark{park_mem[wave], 0};
+        RowParkIds park{park_mem[wave], park_rows[wave], 0};
         half2_t xr[NCH][4];   // ln1(x) for the QKV rows, then ln2(x) for the MLP-up rows
         ln_fetch<NCH>(lns, 0, lane, xr);
-        qkv_rows<NCH, EX>(p, xr, qw, lane, t0, park);
+        qkv_rows<NCH, EX>(p, xr, qw, lane, t0, spark);
+        // the MLP-up tiles of a phase are handed out dynamically within the team; the first tile of the next
+        // pass is requested before the event that ends this one, so the wave is not left without loads in flight
+        // (only when a wave can expect four tiles or more per phase: with fewer, the static shares are
+        // already as fine as the tickets, and the ticket round trips cost more than they balance)
+        TileTeam utm = make_team<kUpRpi>(p, 1, 0, up_phase_rows(CPD, 0, p.F), b, G, wave);
+        const bool dynamic = p.dyn_up > 0 || (p.dyn_up < 0 && utm.ntiles >= 4 * utm.nw);
+        if (dynamic) {
+        TeamTiles<NCH, kUpRpi> ut;
+        team_prefetch<NCH, kUpRpi, EX>(p.w_up, p.H, utm, lane, ut);
         event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], kStreamers, tag);
         trace_mark(p, 2);
         ln_fetch<NCH>(lns, 1, lane, xr);
-        // MLP-up rows in kUpPhases ranges, an event after each; the first tile of the next range is
-        // requested before the event, so the wave is not left without loads in flight
-        RowTile<NCH, kUpRpi> u0;
-        RowWalk uw = row_walk<kUpRpi>(strided, sgw, nsw, 0, up_phase_rows(CPD, 0, p.F));
-        up_prefetch<NCH, EX>(p, uw, lane, u0);
 #pragma unroll
         for (int g = 0; g < kUpPhases; ++g) {
-            up_rows<NCH, EX>(p, xr, uw, lane, u0, park);
+            up_team_rows<NCH, EX>(p, xr, utm, lane, ut, park);
             if (g + 1 < kUpPhases) {
-                uw = row_walk<kUpRpi>(strided, sgw, nsw, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F));
+                utm = make_team<kUpRpi>(p, 2 + g, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F), b, G, wave);
+                team_prefetch<NCH, kUpRpi, EX>(p.w_up, p.H, utm, lane, ut);
+            }
+            event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &q.arrived[1 + g], kStreamers, tag);
+            trace_mark(p, g == kUpPhases - 1 ? 5 : 12);
+        }
+        } else {
+        RowTile<NCH, kUpRpi> u0;
+        RowWalk uw = row_walk<kUpRpi>(false, b * kStreamers + wave, nsw, 0, up_phase_rows(CPD, 0, p.F));
+        up_prefetch<NCH, EX>(p, uw, lane, u0);
+        event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], kStreamers, tag);
+        trace_mark(p, 2);
+        ln_fetch<NCH>(lns, 1, lane, xr);
+#pragma unroll
+        for (int g = 0; g < kUpPhases; ++g) {
+            up_rows<NCH, EX>(p, xr, uw, lane, u0, spark);
+            if (g + 1 < kUpPhases) {
+                uw = row_walk<kUpRpi>(false, b * kStreamers + wave, nsw, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F));
                 up_prefetch<NCH, EX>(p, uw, lane, u0);
             }
             event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &q.arrived[1 + g], kStreamers, tag);
             trace_mark(p, g == kUpPhases - 1 ? 5 : 12);
+        }
         }
     } else {
         // attention wave hw takes the (head, split) items b + (hw + 4 k) G; what does not depend on the QKV
@@ -393,7 +456,7 @@ constexpr size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 long long* g_trace = nullptr;   // see cfpp_debug_set_trace
 
 struct WorkspaceLayout {
-    size_t qkv_raw, attn_vec, inter, part_ml, part_acc, head_cnt, bar, grp, mbox, total;
+    size_t qkv_raw, attn_vec, inter, part_ml, part_acc, head_cnt, bar, grp, mbox, team, total;
 };
 
 WorkspaceLayout workspace_layout(const cfpp_neox_dims& d) {
@@ -409,6 +472,7 @@ WorkspaceLayout workspace_layout(const cfpp_neox_dims& d) {
     w.bar = take(64);
     w.grp = take((size_t)(kBarExit + 1) * kEventGroups * kMailboxInts * 4);
     w.mbox = take((size_t)kMaxGrid * kMailboxInts * 4);
+    w.team = take((size_t)(1 + kUpPhases) * (kMaxGrid / kTeamWgs) * kMailboxInts * 4);
     w.total = off;
     return w;
 }
@@ -574,6 +638,7 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     const int per_head = fused_grid() * kStreamers / (d->heads > 0 ? d->heads : 1);
     if (p.max_split > per_head) p.max_split = per_head < 1 ? 1 : per_head;
     p.row_walk_strided = env_int("CFPP_ROW_WALK_STRIDED", 0);
+    p.dyn_up = env_int("CFPP_DYN_UP", -1);
     char* ws = reinterpret_cast<char*>(workspace);
     p.qkv_raw = reinterpret_cast<float*>(ws + L.qkv_raw);
     p.attn_vec = reinterpret_cast<half_t*>(ws + L.attn_vec);
@@ -584,6 +649,7 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     p.bar = reinterpret_cast<int*>(ws + L.bar);
     p.grp = reinterpret_cast<int*>(ws + L.grp);
     p.mbox = reinterpret_cast<int*>(ws + L.mbox);
+    p.team = reinterpret_cast<int*>(ws + L.team);
     p.c_base0 = p.x; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 1;
     p.trace = g_trace;
     *out = p;
