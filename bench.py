@@ -22,6 +22,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per launch of the fused layer kernel (fetched + written) from the committed hardware-counter
+# summary (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the 256 MiB calibration copy), keyed by
+# (model, context); other workloads have no counter run and report null.
+MEASURED_TRAFFIC_BYTES = {("pythia_6b9", 2048): 439.3e6 + 2.81e6}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -192,7 +197,8 @@ def main():
                                f"batch-1 greedy decode, hipGraph replay, context {args.ctx}",
                    "mode": args.mode, "context": args.ctx, "hidden": cfg.hidden, "ffn": cfg.ffn, "layers": cfg.n_layers},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.model, args.ctx)) if args.mode == "fused" else None,
                      "kernel": "k_fused (one decoder layer)" if args.mode == "fused" else "stage A+B+C kernels (one decoder layer)",
                      "bytes_per_launch": lb, "launch_us": round(lay_ms * 1e3, 2)},
         "step": {"bytes": sb, "hbm_gbps": round(sb / (tpot * 1e-3) / 1e9, 1),
