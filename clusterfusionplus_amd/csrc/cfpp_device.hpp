@@ -70,6 +70,12 @@ struct LayerParams {
     int max_split;      // cap on the KV splits per head (<= kMaxSplit)
     int row_walk_strided;   // streaming waves take interleaved instead of contiguous row ranges
     int dyn_up;             // MLP-up tiles handed out dynamically within teams of workgroups: 1 yes, 0 no, -1 by size
+    // layer family switches (defaults = GPT-NeoX): RMSNorm instead of LayerNorm; where head h's raw q, k, v sit in
+    // qkv_raw (NeoX interleaves [h][q|k|v][D]: stride 3D, offsets D and 2D; LLaMA stacks [q;k;v]: stride D,
+    // offsets H and 2H); whether split 0 appends the new K/V row to the caches
+    int norm_rms, qkv_head_stride, qkv_k_off, qkv_v_off, append_kv;
+    const half_t* x_add;    // nullable: a second input row added to x (fp16-rounded) before the norm ...
+    half_t* x_sum_out;      // ... and where the sum is stored (the caller's residual stream)
     // scratch
     float* qkv_raw;     // [3H] fp32: W_qkv ln1(x) + b_qkv, before RoPE
     half_t* attn_vec;   // [H] fp16: merged attention output (input of the O projection)
@@ -331,46 +337,70 @@ struct LnOwn {
     u32x4 rx[OWN], rw1[OWN], rb1[OWN], rw2[OWN], rb2[OWN];
 };
 
+// What the cooperative norm needs to know about its inputs.
+struct NormSpec {
+    const half_t *x, *x_add;        // input row; optional second row added to it (sum rounded to fp16)
+    half_t* x_sum_out;              // optional: where workgroup 0 stores that sum
+    const half_t *w1, *b1, *w2, *b2;   // affine vectors of slot 0 and (TWO) slot 1; a null bias is zero, a null w2 skips slot 1
+    int H, rms;                     // rms: RMSNorm (no mean subtraction) instead of LayerNorm
+    float eps;
+};
+__device__ __forceinline__ NormSpec norm_spec(const LayerParams& p) {
+    return NormSpec{p.x, p.x_add, p.x_sum_out, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, p.H, p.norm_rms, p.eps};
+}
+
 template <int NCH, int NW, bool TWO>
-__device__ __forceinline__ void ln_coop_load(LnOwn<NCH, NW>& o, const half_t* __restrict__ x, int H,
-                                             const half_t* __restrict__ w1, const half_t* __restrict__ b1,
-                                             const half_t* __restrict__ w2, const half_t* __restrict__ b2, int wave, int lane) {
+__device__ __forceinline__ void ln_coop_load(LnOwn<NCH, NW>& o, const NormSpec& ns, int wave, int lane) {
     const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int k = 0; k < LnOwn<NCH, NW>::OWN; ++k) {
         const int col = (wave + k * NW) * kChunk + lane * 8;
-        const bool in = wave + k * NW < NCH && col < H;
-        o.rx[k] = in ? ld_agent16(x + col) : z;     // written by the previous layer, possibly in this same launch
-        o.rw1[k] = in ? ld16(w1 + col) : z;
-        o.rb1[k] = in ? ld16(b1 + col) : z;
+        const bool in = wave + k * NW < NCH && col < ns.H;
+        o.rx[k] = in ? ld_agent16(ns.x + col) : z;     // written by the previous layer, possibly in this same launch
+        o.rw1[k] = in ? ld16(ns.w1 + col) : z;
+        o.rb1[k] = (in && ns.b1) ? ld16(ns.b1 + col) : z;
         if (TWO) {
-            o.rw2[k] = in ? ld16(w2 + col) : z;
-            o.rb2[k] = in ? ld16(b2 + col) : z;
+            o.rw2[k] = (in && ns.w2) ? ld16(ns.w2 + col) : z;
+            o.rb2[k] = (in && ns.b2) ? ld16(ns.b2 + col) : z;
+        }
+        if (ns.x_add != nullptr) {
+            // x <- fp16(x + x_add), as the reference's fused add + RMSNorm does (reference
+            // include/5090/llama/kernel_sglang.cuh:98-105); workgroup 0 stores the sum
+            const u32x4 ra = in ? ld_agent16(ns.x_add + col) : z;
+            float a[8], b[8];
+            unpack8(o.rx[k], a); unpack8(ra, b);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) a[j] += b[j];
+            o.rx[k] = pack8(a);
+            if (in && ns.x_sum_out != nullptr && blockIdx.x == 0) *reinterpret_cast<u32x4*>(ns.x_sum_out + col) = o.rx[k];
         }
     }
 }
 
 // Every wave of the workgroup must call this (workgroup barriers inside).
 template <int NCH, int NW, bool TWO>
-__device__ __forceinline__ void ln_coop_finish(const LnOwn<NCH, NW>& o, int H, float eps, LnShared<NCH>& sh, int wave, int lane) {
+__device__ __forceinline__ void ln_coop_finish(const LnOwn<NCH, NW>& o, const NormSpec& ns, LnShared<NCH>& sh, int wave, int lane) {
     constexpr int OWN = LnOwn<NCH, NW>::OWN;
-#pragma unroll
-    for (int k = 0; k < OWN; ++k) {
-        const int i = wave + k * NW;
-        if (i < NCH) {
-            float xv[8], s = 0.f;
-            unpack8(o.rx[k], xv);     // lanes past H hold zeros
-#pragma unroll
-            for (int j = 0; j < 8; ++j) s += xv[j];
-            s = wave_sum(s);
-            if (lane == 0) sh.part[0][i] = s;
-        }
-    }
-    __syncthreads();
+    const int H = ns.H;
     float mean = 0.f;
+    if (!ns.rms) {
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) mean += sh.part[0][i];
-    mean /= (float)H;
+        for (int k = 0; k < OWN; ++k) {
+            const int i = wave + k * NW;
+            if (i < NCH) {
+                float xv[8], s = 0.f;
+                unpack8(o.rx[k], xv);     // lanes past H hold zeros
+#pragma unroll
+                for (int j = 0; j < 8; ++j) s += xv[j];
+                s = wave_sum(s);
+                if (lane == 0) sh.part[0][i] = s;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) mean += sh.part[0][i];
+        mean /= (float)H;
+    }
 #pragma unroll
     for (int k = 0; k < OWN; ++k) {
         const int i = wave + k * NW;
@@ -389,7 +419,7 @@ __device__ __forceinline__ void ln_coop_finish(const LnOwn<NCH, NW>& o, int H, f
     float var = 0.f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) var += sh.part[1][i];
-    const float rstd = 1.0f / sqrtf(var / (float)H + eps);
+    const float rstd = 1.0f / sqrtf(var / (float)H + ns.eps);
 #pragma unroll
     for (int k = 0; k < OWN; ++k) {
         const int i = wave + k * NW;
@@ -674,8 +704,9 @@ __device__ __forceinline__ void rope_coeffs(int d0, int rot, const float* __rest
     for (int j = 0; j < 8; ++j) {
         const int d = d0 + j;
         const bool rotd = act && d < rot;
-        rc.c[j] = rotd ? cs[d] : 1.f;
-        rc.sg[j] = rotd ? (d < hr ? -sn[d] : sn[d]) : 0.f;
+        const int t = d < hr ? d : d - hr;       // both halves use the angle of the pair (entries [0, rot/2) of the table)
+        rc.c[j] = rotd ? cs[t] : 1.f;
+        rc.sg[j] = rotd ? (d < hr ? -sn[t] : sn[t]) : 0.f;
     }
 }
 __device__ __forceinline__ void rope_load8(const float* __restrict__ v, int d0, int rot, const RopeCoeffs& rc, bool act,
@@ -752,7 +783,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     const int head = it.head, sp = it.sp, nsplit = it.nsplit, S = it.S, end = it.end;
     const bool act = sub * 8 < D;
     const int d0 = act ? sub * 8 : 0;
-    const float* __restrict__ raw = p.qkv_raw + (size_t)head * 3 * D;
+    const float* __restrict__ raw = p.qkv_raw + (size_t)head * p.qkv_head_stride;
 
     // cos and sin of this position, requested together with q (one round trip)
     RopeCoeffs rc;
@@ -773,15 +804,15 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     // the new token: split 0 owns it (appends it, returns it, and seeds its softmax state with it)
     if (sp == 0 && grp == 0) {
         float kf[8], vf[8];
-        rope_load8(raw + D, d0, p.rot, rc, act, kf);
-        raw_load8(raw + 2 * D, d0, act, vf);
+        rope_load8(raw + p.qkv_k_off, d0, p.rot, rc, act, kf);
+        raw_load8(raw + p.qkv_v_off, d0, act, vf);
         const u32x4 kp = pack8(kf), vp = pack8(vf);
         unpack8(kp, kf); unpack8(vp, vf);      // attend over the fp16 values the cache will hold
         if (act) {
             const size_t o = (size_t)head * D + d0;
             *reinterpret_cast<u32x4*>(p.k_new + o) = kp;
             *reinterpret_cast<u32x4*>(p.v_new + o) = vp;
-            if (S < p.cache_rows) {
+            if (p.append_kv && S < p.cache_rows) {
                 *reinterpret_cast<u32x4*>(p.k_cache + (size_t)S * H + o) = kp;
                 *reinterpret_cast<u32x4*>(p.v_cache + (size_t)S * H + o) = vp;
             }

@@ -59,7 +59,7 @@ __device__ __forceinline__ void qkv_rows(const LayerParams& p, const half2_t (&x
         [&](const RowPark& pk, int k0) {
             if (lane < pk.n) {
                 const int row = walk_row<RPI>(rw, k0 + lane);
-                st_agent(p.qkv_raw + row, pk.slot[lane] + (float)p.b_qkv[row]);
+                st_agent(p.qkv_raw + row, pk.slot[lane] + (p.b_qkv ? (float)p.b_qkv[row] : 0.f));
             }
         });
 }
@@ -113,7 +113,7 @@ __device__ __forceinline__ void qkv_team_rows(const LayerParams& p, const half2_
     gemv_team<NCH, StageARpi<NCH>::value, EX>(p.w_qkv, p.H, tm, x1, lane, tt, park, [&](const RowParkIds& pk) {
         if (lane < pk.n) {
             const int row = pk.row[lane];
-            if (row >= 0) st_agent(p.qkv_raw + row, pk.slot[lane] + (float)p.b_qkv[row]);
+            if (row >= 0) st_agent(p.qkv_raw + row, pk.slot[lane] + (p.b_qkv ? (float)p.b_qkv[row] : 0.f));
         }
     });
 }
@@ -142,11 +142,11 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_a(LayerParams p) {
     const bool strided = p.row_walk_strided != 0;
     const RowWalk qw = row_walk<StageARpi<NCH>::value>(strided, gw, nw, 0, 3 * p.H);
     LnOwn<NCH, kStreamers> own;
-    ln_coop_load<NCH, kStreamers, true>(own, p.x, p.H, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, wave, lane);
+    ln_coop_load<NCH, kStreamers, true>(own, norm_spec(p), wave, lane);
     __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
     RowTile<NCH, StageARpi<NCH>::value> t0;
     qkv_prefetch<NCH, EX>(p, qw, lane, t0);
-    ln_coop_finish<NCH, kStreamers, true>(own, p.H, p.eps, lns, wave, lane);
+    ln_coop_finish<NCH, kStreamers, true>(own, norm_spec(p), lns, wave, lane);
     half2_t xr[NCH][4];
     ln_fetch<NCH>(lns, 0, lane, xr);
     qkv_rows<NCH, EX>(p, xr, qw, lane, t0, park);
@@ -248,8 +248,8 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int l, int n_l
     // LayerNorm by all eight waves
     {
         LnOwn<NCH, kFusedWaves> own;
-        ln_coop_load<NCH, kFusedWaves, true>(own, p.x, p.H, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, wave, lane);
-        ln_coop_finish<NCH, kFusedWaves, true>(own, p.H, p.eps, lns, wave, lane);
+        ln_coop_load<NCH, kFusedWaves, true>(own, norm_spec(p), wave, lane);
+        ln_coop_finish<NCH, kFusedWaves, true>(own, norm_spec(p), lns, wave, lane);
     }
     trace_mark(p, 1);
 
@@ -392,11 +392,12 @@ __global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __res
     const RowWalk rw = row_walk<RPIA>(false, gw, nw, 0, vocab);   // contiguous rows per wave
     __shared__ LnShared<NCH> lns;
     LnOwn<NCH, NWV> own;
-    ln_coop_load<NCH, NWV, false>(own, x, H, ln_w, ln_b, nullptr, nullptr, wave, lane);
+    const NormSpec ns{x, nullptr, nullptr, ln_w, ln_b, nullptr, nullptr, H, 0, eps};
+    ln_coop_load<NCH, NWV, false>(own, ns, wave, lane);
     __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
     RowTile<NCH, RPIA> t0;
     if (rw.ntiles > 0) load_row_tile<NCH, RPIA, EX>(t0, W, H, rw.first, rw.sit, rw.end, lane);
-    ln_coop_finish<NCH, NWV, false>(own, H, eps, lns, wave, lane);
+    ln_coop_finish<NCH, NWV, false>(own, ns, lns, wave, lane);
     half2_t x1[NCH][4];
     ln_fetch<NCH>(lns, 0, lane, x1);
     float bv = -INFINITY;
@@ -701,6 +702,8 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     const int per_head = fused_grid() * kStreamers / (d->heads > 0 ? d->heads : 1);
     if (p.max_split > per_head) p.max_split = per_head < 1 ? 1 : per_head;
     p.row_walk_strided = env_int("CFPP_ROW_WALK_STRIDED", 0);
+    p.norm_rms = 0; p.qkv_head_stride = 3 * d->head_dim; p.qkv_k_off = d->head_dim; p.qkv_v_off = 2 * d->head_dim;
+    p.append_kv = 1; p.x_add = nullptr; p.x_sum_out = nullptr;
     p.dyn_up = env_int("CFPP_DYN_UP", -1);
     char* ws = reinterpret_cast<char*>(workspace);
     p.qkv_raw = reinterpret_cast<float*>(ws + L.qkv_raw);
@@ -792,6 +795,56 @@ int cfpp_neox_attention_mlp_up(const cfpp_neox_dims* dims, const cfpp_neox_weigh
     p.out = reinterpret_cast<half_t*>(io->attn_output);          // stage C: W_o attn + b_o only
     p.c_base0 = nullptr; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 0;
     return run_split(pl, p, seq_hint_of(io), reinterpret_cast<hipStream_t>(stream));
+}
+
+// LLaMA attention block: the NeoX stages with RMSNorm, stacked [q;k;v] rows, whole-head RoPE, no biases, no cache
+// write, no MLP.  Three plain launches (norm + QKV rows, attention items, O projection).
+static cfpp_neox_dims llama_dims(int32_t hidden, int32_t heads, int32_t head_dim, float eps) {
+    // ffn only sizes the (unused) MLP scratch and picks an existing kernel instantiation
+    return cfpp_neox_dims{hidden, heads, head_dim, head_dim, 4 * hidden, eps};
+}
+size_t cfpp_llama_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim) {
+    const cfpp_neox_dims d = llama_dims(hidden, heads, head_dim, 1e-6f);
+    return cfpp_neox_workspace_bytes(&d);
+}
+int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!a || !workspace) return CFPP_ERR_NULL;
+    const cfpp_neox_dims d = llama_dims(a->hidden, a->heads, a->head_dim, a->eps);
+    int rc = check_dims(&d);
+    if (rc) return rc;
+    const void* req[] = {a->rms_w, a->w_qkv, a->w_o, a->input, a->output, a->k_new, a->v_new, a->k_cache, a->v_cache, a->cos, a->sin};
+    for (const void* q : req) {
+        if (!q) return CFPP_ERR_NULL;
+        if (!aligned16(q)) return CFPP_ERR_ALIGN;
+    }
+    if (a->residual && !aligned16(a->residual)) return CFPP_ERR_ALIGN;
+    if (a->seq_len < 0) return CFPP_ERR_SEQ;
+    const WorkspaceLayout L = workspace_layout(d);
+    if (workspace_bytes < L.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CFPP_ERR_WORKSPACE;
+    Plan pl;
+    if ((rc = make_plan(d, &pl))) return rc;
+    if (!shape_supported(pl)) return CFPP_ERR_DIMS;
+
+    // start from the NeoX parameter block of the same geometry, then switch the family-specific parts
+    cfpp_neox_weights w{};
+    w.ln_w = a->rms_w; w.ln_b = a->rms_w; w.w_qkv = a->w_qkv; w.b_qkv = a->rms_w; w.w_o = a->w_o; w.b_o = a->rms_w;
+    w.post_ln_w = a->rms_w; w.post_ln_b = a->rms_w; w.w_up = a->w_qkv; w.b_up = a->rms_w; w.w_down = a->w_qkv; w.b_down = a->rms_w;
+    cfpp_neox_io io{};
+    io.input = a->input; io.output = a->output; io.k_new = a->k_new; io.v_new = a->v_new;
+    io.k_cache = const_cast<void*>(a->k_cache); io.v_cache = const_cast<void*>(a->v_cache);
+    io.cache_rows = a->seq_len; io.cos = a->cos; io.sin = a->sin; io.rope_stride = 0; io.seq_len = a->seq_len;
+    LayerParams p;
+    if ((rc = fill_params(&d, &w, &io, workspace, workspace_bytes, true, true, &p, &pl))) return rc;
+    p.F = 0;                                     // no MLP rows in stage A
+    p.ln_b = nullptr; p.ln2_w = nullptr; p.ln2_b = nullptr; p.b_qkv = nullptr; p.b_o = nullptr;
+    p.w_up = nullptr; p.b_up = nullptr; p.w_down = nullptr; p.b_down = nullptr;
+    p.norm_rms = 1;
+    p.qkv_head_stride = d.head_dim; p.qkv_k_off = d.hidden; p.qkv_v_off = 2 * d.hidden;
+    p.append_kv = 0;
+    p.x_add = reinterpret_cast<const half_t*>(a->residual);
+    p.x_sum_out = reinterpret_cast<half_t*>(a->residual);
+    p.c_base0 = nullptr; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 0;
+    return run_split(pl, p, a->seq_len, reinterpret_cast<hipStream_t>(stream));
 }
 
 int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void* attn_output,

@@ -392,6 +392,50 @@ const Model& kpythia_2b8 = kPythia2b8;
 const Model& kpythia_6b9 = kPythia6b9;
 }  // namespace
 
+// llama_decoder_layer_sglang of the reference (include/pybind.cpp:77-88): returns (output, residual, k, v);
+// `residual` is updated in place (residual += input) as the reference does.
+std::tuple<Tensor, Tensor, Tensor, Tensor> llama_decoder_layer_sglang(Tensor input, Tensor residual, Tensor weight_qkv,
+                                                                      Tensor weight_o, Tensor k_cache, Tensor v_cache,
+                                                                      Tensor rms_input_weight, double eps, Tensor cos, Tensor sin,
+                                                                      int64_t num_heads) {
+    TORCH_CHECK(input.defined() && input.dim() >= 1, "input is undefined");
+    const int64_t H = input.numel();
+    TORCH_CHECK(num_heads > 0 && H % num_heads == 0, "hidden size ", H, " is not a multiple of num_heads ", num_heads);
+    const int64_t D = H / num_heads;
+    check_half(input, "input", H, input);
+    check_half(residual, "residual", H, input);
+    check_half(weight_qkv, "weight_qkv", 3 * H * H, input);
+    check_half(weight_o, "weight_o", H * H, input);
+    check_half(rms_input_weight, "rms_input_weight", H, input);
+    const int64_t rows_k = check_cache(k_cache, "k_cache", H, input);
+    const int64_t rows_v = check_cache(v_cache, "v_cache", H, input);
+    TORCH_CHECK(rows_k == rows_v, "k_cache has ", rows_k, " rows but v_cache has ", rows_v);
+    check_rope(cos, "cos", D / 2, input);
+    check_rope(sin, "sin", D / 2, input);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+    auto opts = input.options();
+    Tensor out = torch::empty({1, H}, opts);
+    Tensor k = torch::empty({1, num_heads, D}, opts);
+    Tensor v = torch::empty({1, num_heads, D}, opts);
+    cfpp_llama_attn a{};
+    a.hidden = (int32_t)H; a.heads = (int32_t)num_heads; a.head_dim = (int32_t)D; a.eps = (float)eps;
+    a.rms_w = rms_input_weight.data_ptr(); a.w_qkv = weight_qkv.data_ptr(); a.w_o = weight_o.data_ptr();
+    a.input = input.data_ptr(); a.residual = residual.data_ptr(); a.output = out.data_ptr();
+    a.k_new = k.data_ptr(); a.v_new = v.data_ptr();
+    // an empty cache has no storage: any valid pointer will do, no row of it is read
+    a.k_cache = rows_k > 0 ? k_cache.data_ptr() : input.data_ptr();
+    a.v_cache = rows_k > 0 ? v_cache.data_ptr() : input.data_ptr();
+    a.seq_len = (int32_t)rows_k;
+    a.cos = cos.data_ptr<float>(); a.sin = sin.data_ptr<float>();
+    const size_t bytes = cfpp_llama_workspace_bytes(a.hidden, a.heads, a.head_dim);
+    TORCH_CHECK(bytes > 0, "unsupported layer dimensions (hidden ", H, ", heads ", num_heads, ")");
+    hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    const cfpp_neox_dims d{a.hidden, a.heads, a.head_dim, a.head_dim, 4 * a.hidden, a.eps};
+    Tensor ws = workspace_for(d, input.device(), st);
+    check_rc(cfpp_llama_attention_decode(&a, ws_ptr(ws), bytes, st), "llama_decoder_layer_sglang");
+    return std::make_tuple(out, residual, k, v);
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "MI355X (gfx950) fused GPT-NeoX / Pythia decode step";
     DEFINE_MODEL_OPS(m, pythia_2b8)
@@ -405,6 +449,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         TORCH_CHECK(cfpp_neox_workspace_bytes(&m.dims) > 0, "unsupported layer dimensions");
         return decoder_layer(m, split ? CFPP_MODE_SPLIT : CFPP_MODE_FUSED, LAYER_PACK(mlp_down_weight, mlp_down_bias), current_seq_len);
     });
+    m.def("llama_decoder_layer_sglang", &llama_decoder_layer_sglang, py::arg("input"), py::arg("residual"), py::arg("weight_qkv"),
+          py::arg("weight_o"), py::arg("k_cache"), py::arg("v_cache"), py::arg("rms_input_weight"), py::arg("eps"), py::arg("cos"),
+          py::arg("sin"), py::arg("num_heads") = 32);
     m.def("cfpp_version", []() { return std::string(cfpp_version()); });
     m.def("debug_set_trace", [](c10::optional<Tensor> buf) {
         // int64 device tensor of at least 1024*16*16 elements, or None to switch tracing off

@@ -106,6 +106,36 @@ int cfpp_neox_layer_decode(const cfpp_neox_dims* dims, const cfpp_neox_weights* 
 int cfpp_neox_attention_mlp_up(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io,
                                void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- LLaMA attention block (sglang flavour) -------------------------------------------------------
+ * r = fp16(input + residual) (stored back into `residual` when it is given; r = input otherwise);
+ * n = RMSNorm(r; eps) * rms_w;  [q;k;v] = W_qkv n with W_qkv [3H, H] = [Wq; Wk; Wv] (not interleaved);
+ * NeoX (rotate-half) RoPE over the whole head on q and k, cos/sin fp32 with >= head_dim/2 entries (the
+ * angles of the pairs);  attention over cache rows [0, seq_len) plus the new token (the caches are NOT
+ * written: k_new / v_new are returned and the caller appends);  output = W_o attn  (no bias, no residual).
+ * Workspace: cfpp_llama_workspace_bytes, 256-byte aligned, zeroed once, one per stream.
+ * Replaces llama_decoder_layer_sglang_sm120 (reference include/pybind.cpp:77-88;
+ * include/5090/llama/llama_kernel_sglang_dispatch.cu:4-160; include/5090/llama/kernel_sglang.cuh). */
+typedef struct cfpp_llama_attn {
+    int32_t hidden, heads, head_dim;
+    float eps;
+    const void* rms_w;       /* [H] fp16 */
+    const void* w_qkv;       /* [3H, H] fp16 */
+    const void* w_o;         /* [H, H] fp16 */
+    const void* input;       /* [H] fp16 */
+    void* residual;          /* [H] fp16, in/out, may be NULL */
+    void* output;            /* [H] fp16 */
+    void* k_new;             /* [heads*D] fp16: rotated K of the new token */
+    void* v_new;             /* [heads*D] fp16 */
+    const void* k_cache;     /* [seq_len, H] fp16, read only */
+    const void* v_cache;
+    int32_t seq_len;         /* cache rows attended */
+    const float* cos;        /* [>= D/2] fp32 */
+    const float* sin;
+} cfpp_llama_attn;
+
+size_t cfpp_llama_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim);
+int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Second half: output = input + attn_output + W_down mlp_intermediate + b_down.
  * Replaces pythia_2b8_mlp_only_sm120 (reference include/pybind.cpp:174-180;
  * pythia_kernel_dispatch_split.cu:364-426). */

@@ -81,3 +81,67 @@ def build_hf_model(dims: NeoxDims, layers: List[Dict[str, torch.Tensor]], embed,
         model.gpt_neox.final_layer_norm.bias.copy_(final_ln_b.to(dtype).reshape(-1))
         model.get_output_embeddings().weight.copy_(lm_head.to(dtype))
     return model
+
+
+# ---- LLaMA (pins llama_layer_decode and llama_attention_sglang) ------------------------------------
+
+def build_hf_llama_layer(dims, w: Dict[str, torch.Tensor], dtype=torch.float32):
+    """HF LlamaDecoderLayer from a local config; `w` as in neox_oracle.llama_layer_decode (missing MLP / rms2
+    entries are left at their random initialisation: the attention-only checks do not use them)."""
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaDecoderLayer
+    H = dims.hidden
+    cfg = LlamaConfig(hidden_size=H, intermediate_size=max(dims.ffn, 8), num_hidden_layers=1, num_attention_heads=dims.heads,
+                      num_key_value_heads=dims.heads, head_dim=dims.head_dim, rms_norm_eps=dims.eps, vocab_size=32,
+                      attention_bias=False, mlp_bias=False, hidden_act="silu", max_position_embeddings=64)
+    cfg._attn_implementation = "eager"
+    layer = LlamaDecoderLayer(cfg, layer_idx=0).to(dtype).eval()
+    f = lambda t: t.detach().cpu().to(dtype)
+    with torch.no_grad():
+        layer.input_layernorm.weight.copy_(f(w["rms1"]).reshape(H))
+        wq, wk, wv = f(w["w_qkv"]).reshape(3, H, H)
+        layer.self_attn.q_proj.weight.copy_(wq); layer.self_attn.k_proj.weight.copy_(wk); layer.self_attn.v_proj.weight.copy_(wv)
+        layer.self_attn.o_proj.weight.copy_(f(w["w_o"]))
+        if "rms2" in w:
+            layer.post_attention_layernorm.weight.copy_(f(w["rms2"]).reshape(H))
+            wg, wu = f(w["w_gate_up"]).reshape(2, dims.ffn, H)
+            layer.mlp.gate_proj.weight.copy_(wg); layer.mlp.up_proj.weight.copy_(wu)
+            layer.mlp.down_proj.weight.copy_(f(w["w_down"]))
+    return layer
+
+
+def _llama_cache(k_cache, v_cache, seq_len, dims, dtype):
+    from transformers import DynamicCache
+    nh, D = dims.heads, dims.head_dim
+    K = k_cache[:seq_len].detach().cpu().to(dtype).reshape(seq_len, nh, D).permute(1, 0, 2)[None].contiguous()
+    V = v_cache[:seq_len].detach().cpu().to(dtype).reshape(seq_len, nh, D).permute(1, 0, 2)[None].contiguous()
+    return DynamicCache(ddp_cache_data=[(K, V)])
+
+
+@torch.no_grad()
+def hf_llama_layer_decode(layer, x, k_cache, v_cache, cos, sin, seq_len: int, dims, dtype=torch.float32):
+    """One decode step through the whole HF LlamaDecoderLayer; returns (output [1,H], k_new, v_new)."""
+    H, D = dims.hidden, dims.head_dim
+    cache = _llama_cache(k_cache, v_cache, seq_len, dims, dtype)
+    c = cos.detach().cpu().to(dtype).reshape(-1)[:D][None, None]
+    s = sin.detach().cpu().to(dtype).reshape(-1)[:D][None, None]
+    out = layer(x.detach().cpu().to(dtype).reshape(1, 1, H), attention_mask=None, past_key_values=cache,
+                position_embeddings=(c, s))
+    if isinstance(out, tuple):
+        out = out[0]
+    return out.reshape(1, H), cache.layers[0].keys[0, :, -1, :][None], cache.layers[0].values[0, :, -1, :][None]
+
+
+@torch.no_grad()
+def hf_llama_attention(layer, r, k_cache, v_cache, cos, sin, dims, dtype=torch.float32):
+    """input_layernorm + self_attn of the HF layer on the (already summed) row r; returns (attn_out [1,H], k_new, v_new)."""
+    H, D = dims.hidden, dims.head_dim
+    S = k_cache.shape[0]
+    cache = _llama_cache(k_cache, v_cache, S, dims, dtype)
+    c = cos.detach().cpu().to(dtype).reshape(-1)[:D][None, None]
+    s = sin.detach().cpu().to(dtype).reshape(-1)[:D][None, None]
+    n = layer.input_layernorm(r.detach().cpu().to(dtype).reshape(1, 1, H))
+    out = layer.self_attn(n, position_embeddings=(c, s), attention_mask=None, past_key_values=cache)
+    if isinstance(out, tuple):
+        out = out[0]
+    return out.reshape(1, H), cache.layers[0].keys[0, :, -1, :][None], cache.layers[0].values[0, :, -1, :][None]

@@ -32,6 +32,8 @@ Parity pinning (what checks this file; see tests/test_oracle_*.py):
   gelu_tanh           pinned  - torch.nn.functional.gelu(approximate="tanh")
   neox_stack_decode   pinned  - HuggingFace GPTNeoXForCausalLM built locally (tiny config)
   llama_layer_decode  pinned  - HuggingFace LlamaDecoderLayer built locally (tiny config)
+  llama_attention_sglang pinned - HuggingFace LlamaRMSNorm + LlamaAttention built locally, S=0 and
+                                zero-W_o closed forms
 """
 from __future__ import annotations
 
@@ -250,6 +252,65 @@ def llama_layer_decode(
     out = _r16(h + inter.reshape(1, -1) @ f(w["w_down"]).t(), round_io)
     return {"output": out, "k_new": k_new[None], "v_new": v_new[None], "attn_output": attn,
             "mlp_intermediate": inter.reshape(-1), "attn_heads": o}
+
+
+def llama_attention_sglang(
+    x: torch.Tensor,
+    residual: Optional[torch.Tensor],
+    w: Dict[str, torch.Tensor],
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    cos: torch.Tensor,
+    sin: torch.Tensor,
+    dims: LlamaDims,
+    dtype: torch.dtype = torch.float32,
+    round_io: bool = True,
+) -> Dict[str, torch.Tensor]:
+    """The attention block the reference fuses for LLaMA (`llama_decoder_layer_sglang`): fused add + RMSNorm,
+    stacked QKV projection, NeoX RoPE over the whole head, attention over every cache row plus the new token
+    (the caches are not written), O projection without bias or residual
+    (reference tests/test_llama.py:57-113; include/5090/llama/kernel_sglang.cuh:97-105 residual add with fp16
+    rounding, :292-293 rope angles cos[d % (D/2)], :332-333 returned k / v;
+    llama_kernel_sglang_dispatch.cu:40 SEQ_LEN = k_cache.size(0)).
+    Weights: `rms1 [H]`, `w_qkv [3H,H]` = [Wq;Wk;Wv], `w_o [H,H]`."""
+    H, nh, D = dims.hidden, dims.heads, dims.head_dim
+    f = lambda t: t.detach().to("cpu").to(dtype)
+    r = f(x).reshape(1, H)
+    if residual is not None:
+        r = _r16(r + f(residual).reshape(1, H), True)        # the sum is an fp16 value in the reference as well
+    n1 = rms_norm(r, f(w["rms1"]).reshape(H), dims.eps)
+    qkv = (n1 @ f(w["w_qkv"]).t()).reshape(3, nh, D)
+    half = D // 2
+    c = f(cos).reshape(-1)[:half]
+    sn = f(sin).reshape(-1)[:half]
+    c2, s2 = torch.cat([c, c]), torch.cat([sn, sn])
+    q = rope_partial_neox(qkv[0], c2, s2, D)
+    k_new = _r16(rope_partial_neox(qkv[1], c2, s2, D), round_io)
+    v_new = _r16(qkv[2], round_io)
+    S = k_cache.shape[0]
+    kc = f(k_cache).reshape(S, nh, D)
+    vc = f(v_cache).reshape(S, nh, D)
+    keys = torch.cat([kc, k_new[None]], dim=0).permute(1, 0, 2)
+    vals = torch.cat([vc, v_new[None]], dim=0).permute(1, 0, 2)
+    p = torch.softmax(torch.einsum("hd,hsd->hs", q, keys) / math.sqrt(D), dim=-1)
+    o = torch.einsum("hs,hsd->hd", p, vals)
+    out = _r16(o.reshape(1, H) @ f(w["w_o"]).t(), round_io)
+    return {"output": out, "residual": r, "k_new": k_new[None], "v_new": v_new[None], "attn_heads": o}
+
+
+def make_llama_attn_inputs(dims: LlamaDims, S: int, seed: int = 0, w_std: float = 0.02):
+    """Seeded fp16 tensors for the LLaMA attention block: weights dict, input, residual, caches [S,H], cos/sin [1,D]
+    (random angles per pair, duplicated halves, as reference tests/test_llama.py:24-28,140-142 builds them)."""
+    H, D = dims.hidden, dims.head_dim
+    g = torch.Generator().manual_seed(7000 + seed)
+    rn = lambda *shape, std=1.0: (torch.randn(*shape, generator=g) * std).half()
+    w = {"rms1": (1 + 0.1 * torch.randn(H, generator=g)).half(), "w_qkv": rn(3 * H, H, std=w_std), "w_o": rn(H, H, std=w_std)}
+    x, res = rn(1, H), rn(1, H)
+    k, v = rn(S, H), rn(S, H)
+    ang = torch.rand(1, D // 2, generator=g) * (2 * math.pi)
+    cos = torch.cat([torch.cos(ang), torch.cos(ang)], dim=-1).float()
+    sin = torch.cat([torch.sin(ang), torch.sin(ang)], dim=-1).float()
+    return w, x, res, k, v, cos, sin
 
 
 # --------------------------------------------------------------------------------------

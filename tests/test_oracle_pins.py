@@ -215,3 +215,57 @@ def test_cache_side_effect():
     assert torch.equal(k[S], r["k_new"].reshape(-1).half()) and torch.equal(v[S], r["v_new"].reshape(-1).half())
     keep = [i for i in range(k.shape[0]) if i != S]
     assert torch.equal(k[keep], k0[keep]) and torch.equal(v[keep], v0[keep])
+
+
+# ---- LLaMA ------------------------------------------------------------------------------------------
+
+def _tiny_llama():
+    dims = O.LlamaDims(hidden=64, heads=4, head_dim=16, ffn=96, eps=1e-6)
+    S = 7
+    w, x, res, k, v, cos, sin = O.make_llama_attn_inputs(dims, S, seed=1, w_std=0.2)
+    g = torch.Generator().manual_seed(77)
+    w["rms2"] = (1 + 0.1 * torch.randn(dims.hidden, generator=g)).half()
+    w["w_gate_up"] = (0.2 * torch.randn(2 * dims.ffn, dims.hidden, generator=g)).half()
+    w["w_down"] = (0.2 * torch.randn(dims.hidden, dims.ffn, generator=g)).half()
+    return dims, S, w, x, res, k, v, cos, sin
+
+
+def test_llama_attention_sglang_matches_hf_llama_attention():
+    """fused add + RMSNorm + stacked QKV + whole-head NeoX RoPE + attention + O projection == HF LlamaRMSNorm + LlamaAttention."""
+    hf = pytest.importorskip("transformers")
+    from oracle import hf_neox
+    dims, S, w, x, res, k, v, cos, sin = _tiny_llama()
+    got = O.llama_attention_sglang(x, res, w, k, v, cos, sin, dims, dtype=torch.float64, round_io=False)
+    r = (x.double() + res.double()).half().double()
+    assert torch.equal(got["residual"], r)
+    layer = hf_neox.build_hf_llama_layer(dims, w, dtype=torch.float64)
+    want, k_new, v_new = hf_neox.hf_llama_attention(layer, r, k, v, cos, sin, dims, dtype=torch.float64)
+    assert torch.allclose(got["output"], want, atol=1e-6, rtol=0)   # HF eager attention takes its softmax in float32
+    # (HF's LlamaRMSNorm works in float32 whatever the module dtype: agreement to float32 rounding)
+    assert torch.allclose(got["k_new"], k_new, atol=1e-6, rtol=0) and torch.allclose(got["v_new"], v_new, atol=1e-6, rtol=0)
+
+
+def test_llama_layer_decode_matches_hf_llama_decoder_layer():
+    hf = pytest.importorskip("transformers")
+    from oracle import hf_neox
+    dims, S, w, x, res, k, v, cos, sin = _tiny_llama()
+    got = O.llama_layer_decode(x, w, k, v, cos, sin, S, dims, dtype=torch.float64, round_io=False)
+    layer = hf_neox.build_hf_llama_layer(dims, w, dtype=torch.float64)
+    want, k_new, v_new = hf_neox.hf_llama_layer_decode(layer, x, k, v, cos, sin, S, dims, dtype=torch.float64)
+    assert torch.allclose(got["output"], want, atol=3e-6, rtol=0)   # HF works in float32 inside RMSNorm and softmax
+    assert torch.allclose(got["k_new"], k_new, atol=1e-6, rtol=0)
+
+
+def test_llama_attention_closed_forms():
+    dims, S, w, x, res, k, v, cos, sin = _tiny_llama()
+    # no cache rows: the only key is the new token, so the head outputs are its V
+    got = O.llama_attention_sglang(x, res, w, k[:0], v[:0], cos, sin, dims, dtype=torch.float64, round_io=False)
+    assert torch.allclose(got["attn_heads"], got["v_new"][0], atol=1e-12, rtol=0)
+    # without a residual the norm sees the input itself
+    got2 = O.llama_attention_sglang(x, None, w, k, v, cos, sin, dims, dtype=torch.float64, round_io=False)
+    assert torch.equal(got2["residual"], x.double())
+    # zero angles: RoPE is the identity, k_new = Wk n
+    one, zero = torch.ones(1, dims.head_dim), torch.zeros(1, dims.head_dim)
+    got3 = O.llama_attention_sglang(x, None, w, k, v, one, zero, dims, dtype=torch.float64, round_io=False)
+    n = O.rms_norm(x.double(), w["rms1"].double(), dims.eps)
+    assert torch.allclose(got3["k_new"].reshape(-1), (n @ w["w_qkv"].double().t()).reshape(3, -1)[1], atol=1e-12, rtol=0)
