@@ -340,13 +340,12 @@ struct LnOwn {
 // What the cooperative norm needs to know about its inputs.
 struct NormSpec {
     const half_t *x, *x_add;        // input row; optional second row added to it (sum rounded to fp16)
-    half_t* x_sum_out;              // optional: where workgroup 0 stores that sum
     const half_t *w1, *b1, *w2, *b2;   // affine vectors of slot 0 and (TWO) slot 1; a null bias is zero, a null w2 skips slot 1
     int H, rms;                     // rms: RMSNorm (no mean subtraction) instead of LayerNorm
     float eps;
 };
 __device__ __forceinline__ NormSpec norm_spec(const LayerParams& p) {
-    return NormSpec{p.x, p.x_add, p.x_sum_out, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, p.H, p.norm_rms, p.eps};
+    return NormSpec{p.x, p.x_add, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, p.H, p.norm_rms, p.eps};
 }
 
 template <int NCH, int NW, bool TWO>
@@ -365,14 +364,14 @@ __device__ __forceinline__ void ln_coop_load(LnOwn<NCH, NW>& o, const NormSpec& 
         }
         if (ns.x_add != nullptr) {
             // x <- fp16(x + x_add), as the reference's fused add + RMSNorm does (reference
-            // include/5090/llama/kernel_sglang.cuh:98-105); workgroup 0 stores the sum
+            // include/5090/llama/kernel_sglang.cuh:98-105).  The sum is stored by stage C, once every
+            // workgroup has read both rows: x_sum_out may be x_add itself.
             const u32x4 ra = in ? ld_agent16(ns.x_add + col) : z;
             float a[8], b[8];
             unpack8(o.rx[k], a); unpack8(ra, b);
 #pragma unroll
             for (int j = 0; j < 8; ++j) a[j] += b[j];
             o.rx[k] = pack8(a);
-            if (in && ns.x_sum_out != nullptr && blockIdx.x == 0) *reinterpret_cast<u32x4*>(ns.x_sum_out + col) = o.rx[k];
         }
     }
 }
@@ -965,6 +964,8 @@ struct StageC {
     const half_t *base0, *base1;
     half_t* out;
     int nrows;
+    const half_t *sum_a, *sum_b;   // optional: sum_out[r] = fp16(sum_a[r] + sum_b[r]) (the residual stream of a fused add + norm)
+    half_t* sum_out;
 };
 
 __device__ __forceinline__ StageC make_stage_c(const LayerParams& p) {
@@ -972,6 +973,7 @@ __device__ __forceinline__ StageC make_stage_c(const LayerParams& p) {
     c.W1 = p.c_use_o ? p.w_o : nullptr;       c.x1 = p.attn_vec; c.bias1 = p.c_use_o ? p.b_o : nullptr;       c.K1 = p.c_use_o ? p.H : 0;
     c.W2 = p.c_use_down ? p.w_down : nullptr; c.x2 = p.inter;    c.bias2 = p.c_use_down ? p.b_down : nullptr; c.K2 = p.c_use_down ? p.F : 0;
     c.base0 = p.c_base0; c.base1 = p.c_base1; c.out = p.out; c.nrows = p.H;
+    c.sum_a = p.x; c.sum_b = p.x_add; c.sum_out = p.x_add ? p.x_sum_out : nullptr;
     return c;
 }
 
@@ -1164,6 +1166,8 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
             if (c.base0) v += (float)ld_agent(c.base0 + r);     // residual inputs and the output cross layers of one launch
             if (c.base1) v += (float)ld_agent(c.base1 + r);
             st_agent(c.out + r, (half_t)v);
+            // every workgroup is past its norm by now (stage C follows the attention, which follows all QKV rows)
+            if (c.sum_out) c.sum_out[r] = (half_t)((float)ld_agent(c.sum_a + r) + (float)ld_agent(c.sum_b + r));
         }
         __syncthreads();
     }

@@ -313,8 +313,10 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int l, int n_l
     {
         const StageC c = make_stage_c(p);
         const bool streamer = wave < kStreamers;
+        // without an MLP-down pass (attention-only layers) all eight waves share the O-projection rows
+        const bool all_o = c.K2 == 0;
         stage_c_rows<NCH, CPD>(
-            c, b, G, shc, streamer, wave, streamer ? -1 : wave - kStreamers, kStreamers, lane,
+            c, b, G, shc, streamer, wave, all_o ? wave : (streamer ? -1 : wave - kStreamers), all_o ? 2 * kStreamers : kStreamers, lane,
             [&](int g) { event_wait(p.mbox, kBarUp + g, tag, status); trace_mark(p, g == 0 ? 6 : 13); },
             [&] { event_wait(p.mbox, kBarHeads, tag, status); trace_mark(p, 7); });
     }
@@ -392,7 +394,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __res
     const RowWalk rw = row_walk<RPIA>(false, gw, nw, 0, vocab);   // contiguous rows per wave
     __shared__ LnShared<NCH> lns;
     LnOwn<NCH, NWV> own;
-    const NormSpec ns{x, nullptr, nullptr, ln_w, ln_b, nullptr, nullptr, H, 0, eps};
+    const NormSpec ns{x, nullptr, ln_w, ln_b, nullptr, nullptr, H, 0, eps};
     ln_coop_load<NCH, NWV, false>(own, ns, wave, lane);
     __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
     RowTile<NCH, RPIA> t0;
@@ -797,8 +799,8 @@ int cfpp_neox_attention_mlp_up(const cfpp_neox_dims* dims, const cfpp_neox_weigh
     return run_split(pl, p, seq_hint_of(io), reinterpret_cast<hipStream_t>(stream));
 }
 
-// LLaMA attention block: the NeoX stages with RMSNorm, stacked [q;k;v] rows, whole-head RoPE, no biases, no cache
-// write, no MLP.  Three plain launches (norm + QKV rows, attention items, O projection).
+// LLaMA attention block: the NeoX kernels with RMSNorm, stacked [q;k;v] rows, whole-head RoPE, no biases, no cache
+// write, no MLP.
 static cfpp_neox_dims llama_dims(int32_t hidden, int32_t heads, int32_t head_dim, float eps) {
     // ffn only sizes the (unused) MLP scratch and picks an existing kernel instantiation
     return cfpp_neox_dims{hidden, heads, head_dim, head_dim, 4 * hidden, eps};
@@ -844,7 +846,11 @@ int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_
     p.x_add = reinterpret_cast<const half_t*>(a->residual);
     p.x_sum_out = reinterpret_cast<half_t*>(a->residual);
     p.c_base0 = nullptr; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 0;
-    return run_split(pl, p, a->seq_len, reinterpret_cast<hipStream_t>(stream));
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const int grid = fused_grid();
+    if (env_int("CFPP_LLAMA_SPLIT", 0) || p.heads > grid * kStreamers) return run_split(pl, p, a->seq_len, st);
+    // one launch: the attention waves fetch their K/V tiles while the streaming waves do the QKV rows
+    return launch_fused(pl, p, grid, st);
 }
 
 int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void* attn_output,
