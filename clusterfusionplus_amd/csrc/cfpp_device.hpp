@@ -76,6 +76,7 @@ struct LayerParams {
     int norm_rms, qkv_head_stride, qkv_k_off, qkv_v_off, append_kv;
     const half_t* x_add;    // nullable: a second input row added to x (fp16-rounded) before the norm ...
     half_t* x_sum_out;      // ... and where the sum is stored (the caller's residual stream)
+    int c_add_sum;          // stage C adds that sum (or x itself when there is no x_add) to the output
     // scratch
     float* qkv_raw;     // [3H] fp32: W_qkv ln1(x) + b_qkv, before RoPE
     half_t* attn_vec;   // [H] fp16: merged attention output (input of the O projection)
@@ -219,6 +220,8 @@ __device__ __forceinline__ float gelu_tanh(float x) {
     return 0.5f * x * (1.0f + t);
 }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// SiLU, x / (1 + e^{-x}), on the native exp2
+__device__ __forceinline__ float silu(float x) { return x / (1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x)); }
 
 // ------------------------------------------------------------------------------------------------
 // device-wide synchronisation (bounded spins; a timeout raises a status flag and falls through)
@@ -966,6 +969,7 @@ struct StageC {
     int nrows;
     const half_t *sum_a, *sum_b;   // optional: sum_out[r] = fp16(sum_a[r] + sum_b[r]) (the residual stream of a fused add + norm)
     half_t* sum_out;
+    int add_sum;                   // ... and the output row gets that sum added (sum_a alone if there is no sum_b)
 };
 
 __device__ __forceinline__ StageC make_stage_c(const LayerParams& p) {
@@ -973,7 +977,7 @@ __device__ __forceinline__ StageC make_stage_c(const LayerParams& p) {
     c.W1 = p.c_use_o ? p.w_o : nullptr;       c.x1 = p.attn_vec; c.bias1 = p.c_use_o ? p.b_o : nullptr;       c.K1 = p.c_use_o ? p.H : 0;
     c.W2 = p.c_use_down ? p.w_down : nullptr; c.x2 = p.inter;    c.bias2 = p.c_use_down ? p.b_down : nullptr; c.K2 = p.c_use_down ? p.F : 0;
     c.base0 = p.c_base0; c.base1 = p.c_base1; c.out = p.out; c.nrows = p.H;
-    c.sum_a = p.x; c.sum_b = p.x_add; c.sum_out = p.x_add ? p.x_sum_out : nullptr;
+    c.sum_a = p.x; c.sum_b = p.x_add; c.sum_out = p.x_add ? p.x_sum_out : nullptr; c.add_sum = p.c_add_sum;
     return c;
 }
 
@@ -1165,9 +1169,15 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
             if (c.bias2) v += (float)c.bias2[r];
             if (c.base0) v += (float)ld_agent(c.base0 + r);     // residual inputs and the output cross layers of one launch
             if (c.base1) v += (float)ld_agent(c.base1 + r);
+            if (c.sum_b != nullptr || c.add_sum) {
+                // the fp16 sum the norm saw; every workgroup is past its norm by now (stage C follows the attention,
+                // which follows all QKV rows), so the sum may overwrite one of its operands
+                float rs = (float)ld_agent(c.sum_a + r);
+                if (c.sum_b != nullptr) rs = (float)(half_t)(rs + (float)ld_agent(c.sum_b + r));
+                if (c.sum_out) c.sum_out[r] = (half_t)rs;
+                if (c.add_sum) v += rs;
+            }
             st_agent(c.out + r, (half_t)v);
-            // every workgroup is past its norm by now (stage C follows the attention, which follows all QKV rows)
-            if (c.sum_out) c.sum_out[r] = (half_t)((float)ld_agent(c.sum_a + r) + (float)ld_agent(c.sum_b + r));
         }
         __syncthreads();
     }

@@ -157,6 +157,35 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_a(LayerParams p) {
     up_rows<NCH, EX>(p, xr, uw, lane, u0, park);
 }
 
+// Norm + gated MLP-up (SwiGLU): inter[r] = silu(Wg[r] . n) * (Wu[r] . n), n = norm(x), with p.w_up = [Wg; Wu] ([2F, H]).
+// A tile is the pair (gate row r, up row r + F); a wave owns a contiguous range of pairs.
+template <int NCH, bool EX>
+__global__ __launch_bounds__(kStreamers * 64) void k_gated_up(LayerParams p) {
+    __shared__ float park_mem[kStreamers][kParkRows];
+    __shared__ LnShared<NCH> lns;
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int gw = blockIdx.x * kStreamers + wave, nw = gridDim.x * kStreamers;
+    RowPark park{park_mem[wave], 0};
+    const int F = p.F;
+    const int first = (int)(((long long)gw * F) / nw), count = (int)(((long long)(gw + 1) * F) / nw) - first;
+    LnOwn<NCH, kStreamers> own;
+    ln_coop_load<NCH, kStreamers, false>(own, norm_spec(p), wave, lane);
+    __builtin_amdgcn_sched_barrier(0);   // the norm inputs go out first
+    RowTile<NCH, 2> t0;
+    if (count > 0) load_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, lane);
+    ln_coop_finish<NCH, kStreamers, false>(own, norm_spec(p), lns, wave, lane);
+    half2_t xr[NCH][4];
+    ln_fetch<NCH>(lns, 0, lane, xr);
+    gemv_tiles<NCH, 2, EX>(
+        p.w_up, p.H, 2 * F, F, count, [=](int t) { return first + t; }, xr, lane, t0, park,
+        [&](const RowPark& pk, int k0) {
+            if (2 * lane + 1 < pk.n) {
+                const int row = first + k0 / 2 + lane;
+                p.inter[row] = (half_t)(silu(pk.slot[2 * lane]) * pk.slot[2 * lane + 1]);
+            }
+        });
+}
+
 // one (head, split) item per wave
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_b(LayerParams p) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
@@ -616,6 +645,19 @@ int launch_fused(const Plan& pl, const LayerParams& p, int grid, hipStream_t st)
 #undef X
     return CFPP_ERR_DIMS;
 }
+template <int NCH>
+int launch_gated_up_t(const LayerParams& p, int grid, hipStream_t st) {
+    if (p.H == NCH * kChunk) hipLaunchKernelGGL((k_gated_up<NCH, true>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
+    else hipLaunchKernelGGL((k_gated_up<NCH, false>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
+    return launch_check();
+}
+int launch_gated_up(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
+#define X(a) if (pl.nch == a) return launch_gated_up_t<a>(p, grid, st);
+    CFPP_NCH_CASES(X)
+#undef X
+    return CFPP_ERR_DIMS;
+}
+
 template <int NCH, int CPD>
 int launch_fused_stack_t(const LayerParams* table, int n_layers, bool exact, int grid, hipStream_t st) {
     const void* fn = exact ? (const void*)(k_fused_stack<NCH, CPD, true>) : (const void*)(k_fused_stack<NCH, CPD, false>);
@@ -705,7 +747,7 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     if (p.max_split > per_head) p.max_split = per_head < 1 ? 1 : per_head;
     p.row_walk_strided = env_int("CFPP_ROW_WALK_STRIDED", 0);
     p.norm_rms = 0; p.qkv_head_stride = 3 * d->head_dim; p.qkv_k_off = d->head_dim; p.qkv_v_off = 2 * d->head_dim;
-    p.append_kv = 1; p.x_add = nullptr; p.x_sum_out = nullptr;
+    p.append_kv = 1; p.x_add = nullptr; p.x_sum_out = nullptr; p.c_add_sum = 0;
     p.dyn_up = env_int("CFPP_DYN_UP", -1);
     char* ws = reinterpret_cast<char*>(workspace);
     p.qkv_raw = reinterpret_cast<float*>(ws + L.qkv_raw);
@@ -846,11 +888,45 @@ int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_
     p.x_add = reinterpret_cast<const half_t*>(a->residual);
     p.x_sum_out = reinterpret_cast<half_t*>(a->residual);
     p.c_base0 = nullptr; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 0;
+    p.c_add_sum = a->add_residual ? 1 : 0;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const int grid = fused_grid();
     if (env_int("CFPP_LLAMA_SPLIT", 0) || p.heads > grid * kStreamers) return run_split(pl, p, a->seq_len, st);
     // one launch: the attention waves fetch their K/V tiles while the streaming waves do the QKV rows
     return launch_fused(pl, p, grid, st);
+}
+
+size_t cfpp_llama_mlp_workspace_bytes(int32_t hidden, int32_t ffn) {
+    if (hidden <= 0 || ffn <= 0 || hidden % 8 || ffn % 8 || hidden > 8 * kChunk) return 0;
+    return align_up((size_t)ffn * 2, 256);
+}
+int cfpp_llama_mlp(const cfpp_llama_mlp_args* m, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!m || !workspace) return CFPP_ERR_NULL;
+    const size_t need = cfpp_llama_mlp_workspace_bytes(m->hidden, m->ffn);
+    if (need == 0 || !(m->eps > 0.f)) return CFPP_ERR_DIMS;
+    if (workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CFPP_ERR_WORKSPACE;
+    const void* req[] = {m->rms_w, m->w_gate_up, m->w_down, m->input, m->output};
+    for (const void* q : req) {
+        if (!q) return CFPP_ERR_NULL;
+        if (!aligned16(q)) return CFPP_ERR_ALIGN;
+    }
+    Plan pl{};
+    pl.nch = (m->hidden + kChunk - 1) / kChunk;
+    pl.cpd = ((m->ffn + kChunk - 1) / kChunk + kStreamers - 1) / kStreamers;
+    if (pl.nch < 1 || pl.nch > 8 || pl.cpd < 1 || pl.cpd > 8 || !shape_supported(pl)) return CFPP_ERR_DIMS;
+    auto h = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
+    LayerParams p{};
+    p.H = m->hidden; p.F = m->ffn; p.eps = m->eps; p.norm_rms = 1;
+    p.x = h(m->input); p.ln_w = h(m->rms_w);
+    p.w_up = h(m->w_gate_up); p.w_down = h(m->w_down);
+    p.inter = reinterpret_cast<half_t*>(workspace);
+    p.out = reinterpret_cast<half_t*>(m->output);
+    p.c_base0 = p.x; p.c_use_o = 0; p.c_use_down = 1;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const int grid = streaming_grid();
+    int rc = launch_gated_up(pl, p, grid, st);
+    if (rc) return rc;
+    return launch_stage_c(pl, p, grid, st);
 }
 
 int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void* attn_output,

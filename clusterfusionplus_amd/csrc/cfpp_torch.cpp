@@ -394,16 +394,16 @@ const Model& kpythia_6b9 = kPythia6b9;
 
 // llama_decoder_layer_sglang of the reference (include/pybind.cpp:77-88): returns (output, residual, k, v);
 // `residual` is updated in place (residual += input) as the reference does.
-std::tuple<Tensor, Tensor, Tensor, Tensor> llama_decoder_layer_sglang(Tensor input, Tensor residual, Tensor weight_qkv,
-                                                                      Tensor weight_o, Tensor k_cache, Tensor v_cache,
-                                                                      Tensor rms_input_weight, double eps, Tensor cos, Tensor sin,
-                                                                      int64_t num_heads) {
+std::tuple<Tensor, Tensor, Tensor> llama_attention_impl(const char* op, Tensor input, c10::optional<Tensor> residual_opt,
+                                                        Tensor weight_qkv, Tensor weight_o, Tensor k_cache, Tensor v_cache,
+                                                        Tensor rms_input_weight, double eps, Tensor cos, Tensor sin,
+                                                        int64_t num_heads, bool add_residual) {
     TORCH_CHECK(input.defined() && input.dim() >= 1, "input is undefined");
     const int64_t H = input.numel();
     TORCH_CHECK(num_heads > 0 && H % num_heads == 0, "hidden size ", H, " is not a multiple of num_heads ", num_heads);
     const int64_t D = H / num_heads;
     check_half(input, "input", H, input);
-    check_half(residual, "residual", H, input);
+    if (residual_opt.has_value()) check_half(*residual_opt, "residual", H, input);
     check_half(weight_qkv, "weight_qkv", 3 * H * H, input);
     check_half(weight_o, "weight_o", H * H, input);
     check_half(rms_input_weight, "rms_input_weight", H, input);
@@ -420,7 +420,8 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> llama_decoder_layer_sglang(Tensor inp
     cfpp_llama_attn a{};
     a.hidden = (int32_t)H; a.heads = (int32_t)num_heads; a.head_dim = (int32_t)D; a.eps = (float)eps;
     a.rms_w = rms_input_weight.data_ptr(); a.w_qkv = weight_qkv.data_ptr(); a.w_o = weight_o.data_ptr();
-    a.input = input.data_ptr(); a.residual = residual.data_ptr(); a.output = out.data_ptr();
+    a.input = input.data_ptr(); a.residual = residual_opt.has_value() ? residual_opt->data_ptr() : nullptr; a.output = out.data_ptr();
+    a.add_residual = add_residual ? 1 : 0;
     a.k_new = k.data_ptr(); a.v_new = v.data_ptr();
     // an empty cache has no storage: any valid pointer will do, no row of it is read
     a.k_cache = rows_k > 0 ? k_cache.data_ptr() : input.data_ptr();
@@ -432,8 +433,55 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> llama_decoder_layer_sglang(Tensor inp
     hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     const cfpp_neox_dims d{a.hidden, a.heads, a.head_dim, a.head_dim, 4 * a.hidden, a.eps};
     Tensor ws = workspace_for(d, input.device(), st);
-    check_rc(cfpp_llama_attention_decode(&a, ws_ptr(ws), bytes, st), "llama_decoder_layer_sglang");
-    return std::make_tuple(out, residual, k, v);
+    check_rc(cfpp_llama_attention_decode(&a, ws_ptr(ws), bytes, st), op);
+    return std::make_tuple(out, k, v);
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> llama_decoder_layer_sglang(Tensor input, Tensor residual, Tensor weight_qkv,
+                                                                      Tensor weight_o, Tensor k_cache, Tensor v_cache,
+                                                                      Tensor rms_input_weight, double eps, Tensor cos, Tensor sin,
+                                                                      int64_t num_heads) {
+    auto r = llama_attention_impl("llama_decoder_layer_sglang", input, residual, weight_qkv, weight_o, k_cache, v_cache,
+                                  rms_input_weight, eps, cos, sin, num_heads, false);
+    return std::make_tuple(std::get<0>(r), residual, std::get<1>(r), std::get<2>(r));
+}
+
+// output = input + W_down (silu(Wg n) * (Wu n)), n = RMSNorm(input) * rms_weight; gate_up_weight = [Wg; Wu] ([2F, H])
+Tensor llama_mlp(Tensor input, Tensor rms_weight, Tensor gate_up_weight, Tensor down_weight, double eps) {
+    TORCH_CHECK(input.defined() && input.dim() >= 1, "input is undefined");
+    const int64_t H = input.numel();
+    check_half(input, "input", H, input);
+    check_half(rms_weight, "rms_weight", H, input);
+    TORCH_CHECK(gate_up_weight.defined() && gate_up_weight.numel() % (2 * H) == 0 && gate_up_weight.numel() > 0,
+                "gate_up_weight must have 2*F*", H, " elements");
+    const int64_t F = gate_up_weight.numel() / (2 * H);
+    check_half(gate_up_weight, "gate_up_weight", 2 * F * H, input);
+    check_half(down_weight, "down_weight", H * F, input);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+    Tensor out = torch::empty({1, H}, input.options());
+    cfpp_llama_mlp_args m{};
+    m.hidden = (int32_t)H; m.ffn = (int32_t)F; m.eps = (float)eps;
+    m.rms_w = rms_weight.data_ptr(); m.w_gate_up = gate_up_weight.data_ptr(); m.w_down = down_weight.data_ptr();
+    m.input = input.data_ptr(); m.output = out.data_ptr();
+    const size_t bytes = cfpp_llama_mlp_workspace_bytes(m.hidden, m.ffn);
+    TORCH_CHECK(bytes > 0, "unsupported MLP dimensions (hidden ", H, ", ffn ", F, ")");
+    hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    // the scratch (one fp16 row of F) comes from torch's caching allocator, which is stream ordered
+    Tensor ws = torch::empty({(int64_t)bytes + 256}, input.options().dtype(torch::kUInt8));
+    check_rc(cfpp_llama_mlp(&m, ws_ptr(ws), bytes, st), "llama_mlp");
+    return out;
+}
+
+// A whole LLaMA layer, batch-1 decode: h = input + attention(RMSNorm(input)); out = h + MLP(RMSNorm(h)).
+// Returns (out, k_new, v_new); the caches are not written.
+std::tuple<Tensor, Tensor, Tensor> llama_decoder_layer_full(Tensor input, Tensor weight_qkv, Tensor weight_o, Tensor k_cache,
+                                                            Tensor v_cache, Tensor rms_input_weight, Tensor rms_post_weight,
+                                                            Tensor gate_up_weight, Tensor down_weight, double eps, Tensor cos,
+                                                            Tensor sin, int64_t num_heads) {
+    auto r = llama_attention_impl("llama_decoder_layer_full", input, c10::nullopt, weight_qkv, weight_o, k_cache, v_cache,
+                                  rms_input_weight, eps, cos, sin, num_heads, true);
+    Tensor out = llama_mlp(std::get<0>(r), rms_post_weight, gate_up_weight, down_weight, eps);
+    return std::make_tuple(out, std::get<1>(r), std::get<2>(r));
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -452,6 +500,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("llama_decoder_layer_sglang", &llama_decoder_layer_sglang, py::arg("input"), py::arg("residual"), py::arg("weight_qkv"),
           py::arg("weight_o"), py::arg("k_cache"), py::arg("v_cache"), py::arg("rms_input_weight"), py::arg("eps"), py::arg("cos"),
           py::arg("sin"), py::arg("num_heads") = 32);
+    m.def("llama_mlp", &llama_mlp, py::arg("input"), py::arg("rms_weight"), py::arg("gate_up_weight"), py::arg("down_weight"),
+          py::arg("eps"));
+    m.def("llama_decoder_layer_full", &llama_decoder_layer_full, py::arg("input"), py::arg("weight_qkv"), py::arg("weight_o"),
+          py::arg("k_cache"), py::arg("v_cache"), py::arg("rms_input_weight"), py::arg("rms_post_weight"),
+          py::arg("gate_up_weight"), py::arg("down_weight"), py::arg("eps"), py::arg("cos"), py::arg("sin"),
+          py::arg("num_heads") = 32);
     m.def("cfpp_version", []() { return std::string(cfpp_version()); });
     m.def("debug_set_trace", [](c10::optional<Tensor> buf) {
         // int64 device tensor of at least 1024*16*16 elements, or None to switch tracing off

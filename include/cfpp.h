@@ -131,10 +131,30 @@ typedef struct cfpp_llama_attn {
     int32_t seq_len;         /* cache rows attended */
     const float* cos;        /* [>= D/2] fp32 */
     const float* sin;
+    int32_t add_residual;    /* 0: output = W_o attn (the reference's op); 1: output = r + W_o attn (the layer's hidden state) */
 } cfpp_llama_attn;
 
 size_t cfpp_llama_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim);
 int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- LLaMA MLP block ---------------------------------------------------------------------------------
+ * output = input + W_down (silu(Wg n) * (Wu n)),  n = RMSNorm(input; eps) * rms_w,  w_gate_up = [Wg; Wu] ([2F, H]),
+ * w_down [H, F].  Two launches (norm + gated up rows, down rows + residual).  The reference fuses only the
+ * attention block of a LLaMA layer (its test leaves the MLP commented out, reference tests/test_llama.py:108-110);
+ * this completes the layer its benchmark configuration describes.
+ * Workspace: cfpp_llama_mlp_workspace_bytes, 256-byte aligned, no initialisation needed, one per stream. */
+typedef struct cfpp_llama_mlp_args {
+    int32_t hidden, ffn;
+    float eps;
+    const void* rms_w;       /* [H] fp16 */
+    const void* w_gate_up;   /* [2F, H] fp16 */
+    const void* w_down;      /* [H, F] fp16 */
+    const void* input;       /* [H] fp16 */
+    void* output;            /* [H] fp16 */
+} cfpp_llama_mlp_args;
+
+size_t cfpp_llama_mlp_workspace_bytes(int32_t hidden, int32_t ffn);
+int cfpp_llama_mlp(const cfpp_llama_mlp_args* m, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Second half: output = input + attn_output + W_down mlp_intermediate + b_down.
  * Replaces pythia_2b8_mlp_only_sm120 (reference include/pybind.cpp:174-180;

@@ -33,7 +33,8 @@ Parity pinning (what checks this file; see tests/test_oracle_*.py):
   neox_stack_decode   pinned  - HuggingFace GPTNeoXForCausalLM built locally (tiny config)
   llama_layer_decode  pinned  - HuggingFace LlamaDecoderLayer built locally (tiny config)
   llama_attention_sglang pinned - HuggingFace LlamaRMSNorm + LlamaAttention built locally, S=0 and
-                                zero-W_o closed forms
+                                zero-angle closed forms
+  llama_mlp           pinned  - through llama_layer_decode (HF LlamaDecoderLayer) and torch silu
 """
 from __future__ import annotations
 
@@ -245,13 +246,25 @@ def llama_layer_decode(
     p = torch.softmax(torch.einsum("hd,hsd->hs", q, keys) / math.sqrt(D), dim=-1)
     o = torch.einsum("hs,hsd->hd", p, vals)
     attn = o.reshape(1, H) @ f(w["w_o"]).t()
-    h = xx + attn
-    n2 = rms_norm(h, f(w["rms2"]).reshape(H), dims.eps)
+    h = _r16(xx + attn, round_io)                      # the hidden state between the two blocks is an fp16 tensor
+    mlp = llama_mlp(h, w, dims, dtype=dtype, round_io=round_io)
+    return {"output": mlp["output"], "k_new": k_new[None], "v_new": v_new[None], "attn_output": attn, "hidden_mid": h,
+            "mlp_intermediate": mlp["mlp_intermediate"], "attn_heads": o}
+
+
+def llama_mlp(h: torch.Tensor, w: Dict[str, torch.Tensor], dims: LlamaDims, dtype: torch.dtype = torch.float32,
+              round_io: bool = True) -> Dict[str, torch.Tensor]:
+    """out = h + Wd (silu(Wg n) * (Wu n)), n = rmsnorm(h) * rms2; `w_gate_up [2F,H]` = [Wg;Wu], `w_down [H,F]`
+    (HF LlamaMLP / LlamaDecoderLayer; the reference's own test leaves this block commented out,
+    reference tests/test_llama.py:108-110)."""
+    H = dims.hidden
+    f = lambda t: t.detach().to("cpu").to(dtype)
+    hh = f(h).reshape(1, H)
+    n2 = rms_norm(hh, f(w["rms2"]).reshape(H), dims.eps)
     gu = (n2 @ f(w["w_gate_up"]).t()).reshape(2, dims.ffn)
     inter = _r16(torch.nn.functional.silu(gu[0]) * gu[1], round_io)
-    out = _r16(h + inter.reshape(1, -1) @ f(w["w_down"]).t(), round_io)
-    return {"output": out, "k_new": k_new[None], "v_new": v_new[None], "attn_output": attn,
-            "mlp_intermediate": inter.reshape(-1), "attn_heads": o}
+    out = _r16(hh + inter.reshape(1, -1) @ f(w["w_down"]).t(), round_io)
+    return {"output": out, "mlp_intermediate": inter.reshape(-1)}
 
 
 def llama_attention_sglang(

@@ -70,3 +70,49 @@ def test_argument_errors(cf):
     with pytest.raises(RuntimeError, match="float32"):
         cf.llama_decoder_layer_sglang(*bad)
     torch.cuda.synchronize()
+
+
+def _full_layer_weights(dims, seed):
+    w, x, res, k, v, cos, sin = O.make_llama_attn_inputs(dims, 0, seed=seed)
+    g = torch.Generator().manual_seed(9000 + seed)
+    w["rms2"] = (1 + 0.1 * torch.randn(dims.hidden, generator=g)).half()
+    w["w_gate_up"] = (0.02 * torch.randn(2 * dims.ffn, dims.hidden, generator=g)).half()
+    w["w_down"] = (0.02 * torch.randn(dims.hidden, dims.ffn, generator=g)).half()
+    return w
+
+
+@pytest.mark.parametrize("hidden,ffn", [(4096, 11008), (1024, 2816)])
+def test_llama_mlp_matches_oracle(cf, hidden, ffn):
+    """output = h + W_down (silu(Wg n) * (Wu n)); ffn 11008 leaves a half-filled last 512-column chunk."""
+    print(f"\ncase llama mlp hidden={hidden} ffn={ffn}", flush=True)
+    dims = O.LlamaDims(hidden=hidden, heads=hidden // 128, head_dim=128, ffn=ffn)
+    w = _full_layer_weights(dims, seed=3)
+    g = torch.Generator().manual_seed(31)
+    h = torch.randn(1, hidden, generator=g).half()
+    ref = O.llama_mlp(h, w, dims)
+    dev = "cuda:0"
+    out = cf.llama_mlp(h.to(dev), w["rms2"].to(dev), w["w_gate_up"].to(dev), w["w_down"].to(dev), dims.eps)
+    torch.cuda.synchronize()
+    assert_close("output", out, ref["output"])
+    # linearity in W_down: doubling it doubles the MLP term (output - h)
+    out2 = cf.llama_mlp(h.to(dev), w["rms2"].to(dev), w["w_gate_up"].to(dev), (w["w_down"].float() * 2).half().to(dev), dims.eps)
+    torch.cuda.synchronize()
+    d1, d2 = out.cpu().float() - h.float(), out2.cpu().float() - h.float()
+    assert float((d2 - 2 * d1).abs().max()) <= 2e-2
+
+
+@pytest.mark.parametrize("S", [4096, 77])
+def test_llama2_7b_full_layer_matches_oracle(cf, S):
+    print(f"\ncase llama2-7b full layer S={S}", flush=True)
+    dims = O.LLAMA2_7B
+    w = _full_layer_weights(dims, seed=4)
+    _, x, _, k, v, cos, sin = O.make_llama_attn_inputs(dims, S, seed=40 + S)
+    ref = O.llama_layer_decode(x, w, k, v, cos, sin, S, dims)
+    dev = "cuda:0"
+    out, kn, vn = cf.llama_decoder_layer_full(x.to(dev), w["w_qkv"].to(dev), w["w_o"].to(dev), k.to(dev), v.to(dev),
+                                              w["rms1"].to(dev), w["rms2"].to(dev), w["w_gate_up"].to(dev), w["w_down"].to(dev),
+                                              dims.eps, cos.to(dev), sin.to(dev), dims.heads)
+    torch.cuda.synchronize()
+    assert_close("output", out, ref["output"])
+    assert_close("k_new", kn, ref["k_new"])
+    assert_close("v_new", vn, ref["v_new"])
