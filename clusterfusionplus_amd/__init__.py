@@ -14,21 +14,27 @@ without the built native libraries raises ImportError (build them with
 """
 import importlib
 import os as _os
-
-import torch as _torch  # noqa: F401  (loads the HIP runtime the native libraries bind to)
+import sys as _sys
 
 _here = _os.path.dirname(_os.path.abspath(__file__))
-for _need in ("libcfpp.so", "_clusterfusion.so"):
-    if not _os.path.exists(_os.path.join(_here, _need)):
-        raise ImportError(
-            f"clusterfusionplus_amd: native library {_need} is missing from {_here}; "
-            "run `python -m clusterfusionplus_amd.build` (needs hipcc for gfx950). There is no fallback path.")
+_missing = [n for n in ("libcfpp.so", "_clusterfusion.so") if not _os.path.exists(_os.path.join(_here, n))]
+# `python -m clusterfusionplus_amd.build` has to get past this file on a fresh checkout: for that one command
+# the package imports without its operators; every other import without the libraries fails here.
+_building = "clusterfusionplus_amd.build" in getattr(_sys, "orig_argv", [])
 
-_native = importlib.import_module("clusterfusionplus_amd._clusterfusion")
+if _missing and not _building:
+    raise ImportError(
+        f"clusterfusionplus_amd: native library {_missing[0]} is missing from {_here}; "
+        "run `python -m clusterfusionplus_amd.build` (needs hipcc for gfx950). There is no fallback path.")
 
-__all__ = [n for n in dir(_native) if not n.startswith("_")]
-globals().update({n: getattr(_native, n) for n in __all__})
+__all__ = []
+if not _missing:
+    import torch as _torch  # noqa: F401  (loads the HIP runtime the native libraries bind to)
 
-from .model import NeoxConfig, PYTHIA_2B8, PYTHIA_6B9, NeoxDecoder, layer_tensor_order, rope_tables  # noqa: E402
+    _native = importlib.import_module("clusterfusionplus_amd._clusterfusion")
+    __all__ = [n for n in dir(_native) if not n.startswith("_")]
+    globals().update({n: getattr(_native, n) for n in __all__})
 
-__all__ += ["NeoxConfig", "PYTHIA_2B8", "PYTHIA_6B9", "NeoxDecoder", "layer_tensor_order", "rope_tables"]
+    from .model import NeoxConfig, PYTHIA_2B8, PYTHIA_6B9, NeoxDecoder, layer_tensor_order, rope_tables  # noqa: E402
+
+    __all__ += ["NeoxConfig", "PYTHIA_2B8", "PYTHIA_6B9", "NeoxDecoder", "layer_tensor_order", "rope_tables"]
