@@ -95,23 +95,14 @@ struct LayerParams {
     long long* trace;   // debugging: per-workgroup phase timestamps of the fused kernel (null = off)
 };
 
-// threadIdx.x behind a compiler barrier: the value is recomputed where it is used.  (When the layers of
-// a stack run in a loop, the compiler otherwise evaluates every thread-dependent address once, in front of
-// the loop, and keeps all of them in registers it does not have.)
-__device__ __forceinline__ int thread_index() {
-    int t = threadIdx.x;
-    asm volatile("" : "+v"(t));
-    return t;
-}
-
 constexpr int kTraceSlots = 16;
 __device__ __forceinline__ void trace_value(const LayerParams& p, int slot, long long v) {
-    if (p.trace != nullptr && (thread_index() & 63) == 0)
-        p.trace[((size_t)blockIdx.x * kMaxWaves + (thread_index() >> 6)) * kTraceSlots + slot] = v;
+    if (p.trace != nullptr && (threadIdx.x & 63) == 0)
+        p.trace[((size_t)blockIdx.x * kMaxWaves + (threadIdx.x >> 6)) * kTraceSlots + slot] = v;
 }
 __device__ __forceinline__ void trace_mark(const LayerParams& p, int slot) {
-    if (p.trace != nullptr && (thread_index() & 63) == 0)
-        p.trace[((size_t)blockIdx.x * kMaxWaves + (thread_index() >> 6)) * kTraceSlots + slot] = wall_clock64();
+    if (p.trace != nullptr && (threadIdx.x & 63) == 0)
+        p.trace[((size_t)blockIdx.x * kMaxWaves + (threadIdx.x >> 6)) * kTraceSlots + slot] = wall_clock64();
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -142,9 +133,6 @@ __device__ __forceinline__ void st_agent2(float* p, float a, float b) {   // p 8
     __hip_atomic_store(reinterpret_cast<uint64_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ float ld_agent(const float* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ half_t ld_agent(const half_t* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void ld_agent2(const float* p, float& a, float& b) {   // p 8-byte aligned
@@ -256,7 +244,7 @@ __device__ __forceinline__ int* group_counter(int* grp, int event, int g) {
 // the one that completes the event writes `tag` into mailbox slot `event` of all `nwg` workgroups and
 // returns true.
 __device__ __forceinline__ bool event_arrive(int* bar, int* grp, int* mbox, int event, int nwg, int* lds_ctr, int per_wg, int tag) {
-    const int lane = thread_index() & 63;
+    const int lane = threadIdx.x & 63;
     drain_memory_ops();
     int go = 1;
     if (lds_ctr != nullptr) {
@@ -290,7 +278,7 @@ __device__ __forceinline__ bool event_arrive(int* bar, int* grp, int* mbox, int 
 // arrivals must be read with ld_agent / ld_agent16.  A wait that expires raises a status flag and
 // falls through.
 __device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, int* status) {
-    if ((thread_index() & 63) == 0) {
+    if ((threadIdx.x & 63) == 0) {
         const int* f = mbox + blockIdx.x * kMailboxInts + slot;
         int spins = 0;
         while (counter_peek(f) != tag) {
@@ -305,7 +293,7 @@ __device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, i
 __device__ __forceinline__ int load_seq_len(const LayerParams& p) {
     int S = p.d_seq_len ? *p.d_seq_len : p.seq_len;
     if (S < 0 || S > p.cache_rows) {
-        if (thread_index() == 0 && blockIdx.x == 0) raise_status(p.bar + kBarStatus, kStatusSeq);
+        if (threadIdx.x == 0 && blockIdx.x == 0) raise_status(p.bar + kBarStatus, kStatusSeq);
         S = S < 0 ? 0 : p.cache_rows;
     }
     return S;
@@ -358,7 +346,7 @@ __device__ __forceinline__ void ln_coop_load(LnOwn<NCH, NW>& o, const NormSpec& 
     for (int k = 0; k < LnOwn<NCH, NW>::OWN; ++k) {
         const int col = (wave + k * NW) * kChunk + lane * 8;
         const bool in = wave + k * NW < NCH && col < ns.H;
-        o.rx[k] = in ? ld_agent16(ns.x + col) : z;     // written by the previous layer, possibly in this same launch
+        o.rx[k] = in ? ld16(ns.x + col) : z;
         o.rw1[k] = in ? ld16(ns.w1 + col) : z;
         o.rb1[k] = (in && ns.b1) ? ld16(ns.b1 + col) : z;
         if (TWO) {
@@ -369,7 +357,7 @@ __device__ __forceinline__ void ln_coop_load(LnOwn<NCH, NW>& o, const NormSpec& 
             // x <- fp16(x + x_add), as the reference's fused add + RMSNorm does (reference
             // include/5090/llama/kernel_sglang.cuh:98-105).  The sum is stored by stage C, once every
             // workgroup has read both rows: x_sum_out may be x_add itself.
-            const u32x4 ra = in ? ld_agent16(ns.x_add + col) : z;
+            const u32x4 ra = in ? ld16(ns.x_add + col) : z;
             float a[8], b[8];
             unpack8(o.rx[k], a); unpack8(ra, b);
 #pragma unroll
@@ -745,7 +733,7 @@ __device__ __forceinline__ void raw_load8(const float* __restrict__ v, int d0, b
 // `sub` of a group holds dims 8 sub .. 8 sub + 7 of its row (lanes with 8 sub >= D contribute nothing).
 // A tile is kAttnT rows per group (32 rows per wave).  An item is a chain of dependent memory round
 // trips, so everything that does not depend on this layer's QKV rows is requested ahead of them by
-// attn_prefetch: the first two K/V tiles.  In the fused kernel that happens while
+// attn_prefetch: the first two K/V tiles and the RoPE coefficients.  In the fused kernel that happens while
 // the attention waves would otherwise sit waiting for the QKV rows.
 constexpr int kAttnT = 8;
 constexpr int kAttnTileRows = 4 * kAttnT;
@@ -753,6 +741,7 @@ struct KvTile { u32x4 k[kAttnT], v[kAttnT]; };
 struct AttnItem {
     int head, sp, nsplit, S, begin, end, ntiles;
     KvTile t0, t1;
+    RopeCoeffs rc;
 };
 // tile i of the item; rows past the end re-read the last row (masked when used): no conditional loads
 __device__ __forceinline__ void attn_load_tile(const LayerParams& p, const AttnItem& it, KvTile& kv, int i, int lane) {
@@ -776,6 +765,11 @@ __device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it
     it.ntiles = it.begin < it.end ? (it.end - it.begin + kAttnTileRows - 1) / kAttnTileRows : 0;
     if (it.ntiles > 0) attn_load_tile(p, it, it.t0, 0, lane);
     if (it.ntiles > 1) attn_load_tile(p, it, it.t1, 1, lane);
+    const int sub = lane & 15;
+    const bool act = sub * 8 < p.D;
+    const float* __restrict__ cs = p.cos + (size_t)S * p.rope_stride;   // stride 0: the row is the position
+    const float* __restrict__ sn = p.sin + (size_t)S * p.rope_stride;
+    rope_coeffs(act ? sub * 8 : 0, p.rot, cs, sn, act, it.rc);
 }
 
 // nwg_to_signal > 0 (fused kernel): a completed head counts towards the kBarHeads event of that many workgroups.
@@ -787,13 +781,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     const int d0 = act ? sub * 8 : 0;
     const float* __restrict__ raw = p.qkv_raw + (size_t)head * p.qkv_head_stride;
 
-    // cos and sin of this position, requested together with q (one round trip)
-    RopeCoeffs rc;
-    {
-        const float* __restrict__ cs = p.cos + (size_t)S * p.rope_stride;   // stride 0: the row is the position
-        const float* __restrict__ sn = p.sin + (size_t)S * p.rope_stride;
-        rope_coeffs(d0, p.rot, cs, sn, act, rc);
-    }
+    const RopeCoeffs& rc = it.rc;
     float q[8];
     rope_load8(raw, d0, p.rot, rc, act, q);
 #pragma unroll
@@ -1153,7 +1141,7 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
         }
         first = false;
         __syncthreads();
-        const int t = thread_index();
+        const int t = threadIdx.x;
         if (t < b1 - b0) {
             const int r = b0 + t;
             float v = 0.f;
@@ -1167,17 +1155,17 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
             if (c.K1 > 0) v += sh.red_o[t];
             if (c.bias1) v += (float)c.bias1[r];
             if (c.bias2) v += (float)c.bias2[r];
-            if (c.base0) v += (float)ld_agent(c.base0 + r);     // residual inputs and the output cross layers of one launch
-            if (c.base1) v += (float)ld_agent(c.base1 + r);
+            if (c.base0) v += (float)c.base0[r];
+            if (c.base1) v += (float)c.base1[r];
             if (c.sum_b != nullptr || c.add_sum) {
                 // the fp16 sum the norm saw; every workgroup is past its norm by now (stage C follows the attention,
                 // which follows all QKV rows), so the sum may overwrite one of its operands
-                float rs = (float)ld_agent(c.sum_a + r);
-                if (c.sum_b != nullptr) rs = (float)(half_t)(rs + (float)ld_agent(c.sum_b + r));
+                float rs = (float)c.sum_a[r];
+                if (c.sum_b != nullptr) rs = (float)(half_t)(rs + (float)c.sum_b[r]);
                 if (c.sum_out) c.sum_out[r] = (half_t)rs;
                 if (c.add_sum) v += rs;
             }
-            st_agent(c.out + r, (half_t)v);
+            c.out[r] = (half_t)v;
         }
         __syncthreads();
     }

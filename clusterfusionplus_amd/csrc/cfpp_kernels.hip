@@ -226,10 +226,6 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
 struct FusedShared { int arrived[1 + kUpPhases]; };
 
 
-// With a table of layers the launch runs them one after the other (layer l reads the hidden state layer
-// l-1 wrote): the kBarExit event of a layer then carries mailbox flags, and every wave waits for it with
-// its first weight tile (streaming waves) or K/V tiles (attention waves) of the next layer already
-// requested, so the launch gap, the cold start and most of the LayerNorm latency of a layer disappear.
 template <int NCH>
 struct FusedLds {
     FusedShared q;
@@ -239,47 +235,43 @@ struct FusedLds {
     int park_rows[kStreamers][kParkRows];
 };
 
-// Layer l of n_layers of one launch; `gen` is the launch generation read at its start.
+// One layer; `gen` is the launch generation read at the start of the launch.
 template <int NCH, int CPD, bool EX>
-__device__ __forceinline__ void fused_layer(const LayerParams& p, int l, int n_layers, int gen, FusedLds<NCH>& lds) {
+__device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, FusedLds<NCH>& lds) {
     FusedShared& q = lds.q;
     StageCShared& shc = lds.shc;
     LnShared<NCH>& lns = lds.lns;
     float (&park_mem)[kStreamers][kParkRows] = lds.park_mem;
     int (&park_rows)[kStreamers][kParkRows] = lds.park_rows;
-    const int lane = thread_index() & 63, wave = first_lane(thread_index() >> 6);   // wave index in a scalar register
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int G = gridDim.x, b = blockIdx.x;
     const int nsw = G * kStreamers;                 // streaming waves in the grid
     int* status = p.bar + kBarStatus;
-    if (thread_index() <= kUpPhases) q.arrived[thread_index()] = 0;
+    if (threadIdx.x <= kUpPhases) q.arrived[threadIdx.x] = 0;
     __syncthreads();
     trace_mark(p, 0);
     trace_value(p, 8, __builtin_amdgcn_s_getreg((3 << 11) | 20));   // XCC_ID: which XCD this workgroup runs on
     trace_value(p, 11, __builtin_amdgcn_s_getreg((31 << 11) | 4));  // HW_ID: wave slot, SIMD, CU, SE
 
-    const int S = load_seq_len(p);
-    const int nsplit = effective_split(p, S);
-    const int nitems = p.heads * nsplit;
-    const int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
-    // what does not depend on the previous layer goes out first: the first QKV tile of a streaming wave;
-    // the first K/V tiles and RoPE coefficients of an attention wave, which takes the (head, split) item
-    // b + hw G (the host caps the KV splits so that no wave has more than one item: attn_count <= kStreamers)
+    // LayerNorm by all eight waves.  Its (few) loads go out first; behind them the first QKV tile of a streaming
+    // wave, so that it is on its way while the statistics are computed
     constexpr int kFusedWaves = 2 * kStreamers;
     constexpr int RPIA = StageARpi<NCH>::value;
     const RowWalk qw = row_walk<RPIA>(false, b * kStreamers + wave, nsw, 0, 3 * p.H);     // streaming waves only
     const int hw = wave - kStreamers;
     RowTile<NCH, RPIA> t0;
-    AttnItem it;
-    if (wave < kStreamers) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
-    else if (hw < attn_count) attn_prefetch(p, it, (b + hw * G) / nsplit, (b + hw * G) % nsplit, nsplit, S, lane);
-    const int tag = first_lane(gen) + 1 + l;
-    if (l > 0) event_wait(p.mbox, kBarExit, tag - 1, status);
-    // LayerNorm by all eight waves
     {
         LnOwn<NCH, kFusedWaves> own;
         ln_coop_load<NCH, kFusedWaves, true>(own, norm_spec(p), wave, lane);
+        __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
+        if (wave < kStreamers) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
         ln_coop_finish<NCH, kFusedWaves, true>(own, norm_spec(p), lns, wave, lane);
     }
+    const int tag = first_lane(gen) + 1;
+    const int S = load_seq_len(p);
+    const int nsplit = effective_split(p, S);
+    const int nitems = p.heads * nsplit;
+    const int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
     trace_mark(p, 1);
 
     if (wave < kStreamers) {
@@ -329,7 +321,12 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int l, int n_l
             }
         }
     } else {
+        // an attention wave takes the (head, split) item b + hw G (the host caps the KV splits so that no wave has
+        // more than one item: attn_count <= kStreamers); what does not depend on the QKV rows (first K/V tiles,
+        // RoPE coefficients) is requested before waiting for them
         if (hw < attn_count) {
+            AttnItem it;
+            attn_prefetch(p, it, (b + hw * G) / nsplit, (b + hw * G) % nsplit, nsplit, S, lane);
             event_wait(p.mbox, kBarQkv, tag, status);
             __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
             trace_mark(p, 3);
@@ -350,12 +347,10 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int l, int n_l
             [&] { event_wait(p.mbox, kBarHeads, tag, status); trace_mark(p, 7); });
     }
     trace_mark(p, 10);
-    // end of the layer (wave 0 stored the output rows of this workgroup): between layers the event tells every
-    // workgroup; after the last one it publishes the new generation, so the flags of this launch turn stale
+    // the last workgroup to leave publishes the new generation: the flags of this launch turn stale
     if (wave == 0) {
-        const bool more = l + 1 < n_layers;
-        const bool last = event_arrive(p.bar, p.grp, more ? p.mbox : nullptr, kBarExit, G, nullptr, 1, tag);
-        if (!more && last && lane == 0) __hip_atomic_store(p.bar + kBarGen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1, tag);
+        if (last && lane == 0) __hip_atomic_store(p.bar + kBarGen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -363,37 +358,9 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int l, int n_l
 template <int NCH, int CPD, bool EX>
 __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     __shared__ FusedLds<NCH> lds;
-    // the flag value of layer l of a launch is gen + 1 + l: requested first, needed at the first event
+    // the flag value of this launch is gen + 1: requested first, needed at the first event
     const int gen = counter_peek(p.bar + kBarGen);
-    fused_layer<NCH, CPD, EX>(p, 0, 1, gen, lds);
-}
-
-// Pointers read from a table in memory are generic as far as the compiler knows, and every access through
-// them would be a flat load; a round trip through the global address space tells it where they point.
-template <class T>
-__device__ __forceinline__ T* as_global(T* q) {
-    return (T*)(__attribute__((address_space(1))) T*)q;
-}
-
-// a stack of layers (same dims, same workspace), parameters in a device-resident table
-template <int NCH, int CPD, bool EX>
-__global__ __launch_bounds__(2 * kStreamers * 64) void k_fused_stack(const LayerParams* __restrict__ table, int n_layers) {
-    __shared__ FusedLds<NCH> lds;
-    const int gen = counter_peek(as_global(table[0].bar) + kBarGen);
-    for (int l = 0; l < n_layers; ++l) {
-        LayerParams p = table[l];
-        p.ln_w = as_global(p.ln_w); p.ln_b = as_global(p.ln_b); p.w_qkv = as_global(p.w_qkv); p.b_qkv = as_global(p.b_qkv);
-        p.w_o = as_global(p.w_o); p.b_o = as_global(p.b_o); p.ln2_w = as_global(p.ln2_w); p.ln2_b = as_global(p.ln2_b);
-        p.w_up = as_global(p.w_up); p.b_up = as_global(p.b_up); p.w_down = as_global(p.w_down); p.b_down = as_global(p.b_down);
-        p.x = as_global(p.x); p.out = as_global(p.out); p.k_new = as_global(p.k_new); p.v_new = as_global(p.v_new);
-        p.k_cache = as_global(p.k_cache); p.v_cache = as_global(p.v_cache);
-        p.cos = as_global(p.cos); p.sin = as_global(p.sin); p.d_seq_len = as_global(p.d_seq_len);
-        p.qkv_raw = as_global(p.qkv_raw); p.attn_vec = as_global(p.attn_vec); p.inter = as_global(p.inter);
-        p.part_ml = as_global(p.part_ml); p.part_acc = as_global(p.part_acc); p.head_cnt = as_global(p.head_cnt);
-        p.bar = as_global(p.bar); p.grp = as_global(p.grp); p.mbox = as_global(p.mbox); p.team = as_global(p.team);
-        p.c_base0 = as_global(p.c_base0); p.c_base1 = as_global(p.c_base1); p.trace = as_global(p.trace);
-        fused_layer<NCH, CPD, EX>(p, l, n_layers, gen, lds);
-    }
+    fused_layer<NCH, CPD, EX>(p, gen, lds);
 }
 
 // ---- whole-model helpers -----------------------------------------------------------------------
@@ -658,19 +625,6 @@ int launch_gated_up(const Plan& pl, const LayerParams& p, int grid, hipStream_t 
     return CFPP_ERR_DIMS;
 }
 
-template <int NCH, int CPD>
-int launch_fused_stack_t(const LayerParams* table, int n_layers, bool exact, int grid, hipStream_t st) {
-    const void* fn = exact ? (const void*)(k_fused_stack<NCH, CPD, true>) : (const void*)(k_fused_stack<NCH, CPD, false>);
-    void* args[] = {&table, &n_layers};
-    CFPP_HIP(hipLaunchKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st));
-    return CFPP_OK;
-}
-int launch_fused_stack(const Plan& pl, const LayerParams* table, int n_layers, bool exact, int grid, hipStream_t st) {
-#define X(a, b) if (pl.nch == a && pl.cpd == b) return launch_fused_stack_t<a, b>(table, n_layers, exact, grid, st);
-    CFPP_SHAPE_CASES(X)
-#undef X
-    return CFPP_ERR_DIMS;
-}
 bool shape_supported(const Plan& pl) {
 #define X(a, b) if (pl.nch == a && pl.cpd == b) return true;
     CFPP_SHAPE_CASES(X)
@@ -1122,7 +1076,6 @@ struct cfpp_neox_stack {
     int hist_cap = 0;
     void* ws = nullptr;
     size_t ws_bytes = 0;
-    LayerParams* table = nullptr;      // device: the layers' parameters, for the one-launch stack kernel (fused mode)
     hipStream_t own_stream = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
@@ -1157,15 +1110,9 @@ int stack_enqueue_step(cfpp_neox_stack* s, hipStream_t st) {
                        reinterpret_cast<const half_t*>(s->desc.embed), s->state, H, s->desc.vocab, s->hidden[0]);
     int rc = launch_check();
     if (rc) return rc;
-    if (s->table) {
-        // all layers in one launch
-        rc = launch_fused_stack(s->plan, s->table, s->desc.n_layers, d.hidden == s->plan.nch * kChunk, fused_grid(), st);
+    for (int l = 0; l < s->desc.n_layers; ++l) {
+        rc = stack_enqueue_layer(s, l, st);
         if (rc) return rc;
-    } else {
-        for (int l = 0; l < s->desc.n_layers; ++l) {
-            rc = stack_enqueue_layer(s, l, st);
-            if (rc) return rc;
-        }
     }
     rc = launch_lm_head(H, s->desc.vocab, d.eps, s->hidden[s->desc.n_layers & 1], s->desc.final_ln_w, s->desc.final_ln_b,
                         s->desc.lm_head, s->logits, s->best_val, s->best_idx, s->grid, st);
@@ -1220,28 +1167,6 @@ int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out) {
     s->best_idx = reinterpret_cast<int*>(s->slab + o_bi);
     s->history = reinterpret_cast<int*>(s->slab + o_hist);
     s->ws = s->slab + o_ws;
-    // Experimental (CFPP_STACK_ONE_LAUNCH=1): all layers of a token in one launch of k_fused_stack.  It gives the
-    // same results, but so far it is slower than one launch per layer: the device-wide event between two
-    // layers costs more than the launch gap it replaces.
-    if (desc->mode == CFPP_MODE_FUSED && env_int("CFPP_STACK_ONE_LAUNCH", 0) && d.heads <= fused_grid() * kStreamers) {
-        std::vector<LayerParams> host(desc->n_layers);
-        for (int l = 0; l < desc->n_layers && rc == CFPP_OK; ++l) {
-            const cfpp_neox_io io = stack_layer_io(s, l);
-            Plan pl;
-            rc = fill_params(&d, &s->layers[l], &io, s->ws, s->ws_bytes, true, true, &host[l], &pl);
-        }
-        if (rc == CFPP_OK) {
-            e = hipMalloc(reinterpret_cast<void**>(&s->table), host.size() * sizeof(LayerParams));
-            if (e == hipSuccess) e = hipMemcpy(s->table, host.data(), host.size() * sizeof(LayerParams), hipMemcpyHostToDevice);
-            if (e != hipSuccess) rc = (int)e;
-        }
-        if (rc != CFPP_OK) {
-            if (s->table) (void)hipFree(s->table);
-            (void)hipFree(s->slab);
-            delete s;
-            return rc;
-        }
-    }
     *out = s;
     return CFPP_OK;
 }
@@ -1346,7 +1271,6 @@ int cfpp_stack_destroy(cfpp_neox_stack* s) {
     if (s->exec) (void)hipGraphExecDestroy(s->exec);
     if (s->graph) (void)hipGraphDestroy(s->graph);
     if (s->own_stream) (void)hipStreamDestroy(s->own_stream);
-    if (s->table) (void)hipFree(s->table);
     if (s->slab) (void)hipFree(s->slab);
     delete s;
     return CFPP_OK;
