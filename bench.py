@@ -120,12 +120,67 @@ def cpu_baseline(cfg, S, budget_s=12.0):
     }
 
 
+def bench_llama_layer(args):
+    """Extra workload (not the headline): one LLaMA-2-7B layer, batch-1 decode at context --ctx (default 4096):
+    the attention block (the reference's llama_decoder_layer_sglang) followed by the MLP block, replayed from a
+    captured graph over 8 weight sets so that every launch reads HBM-cold weights."""
+    import torch
+    import clusterfusion as cf
+    from oracle import neox_oracle as O      # seeded synthetic inputs only
+    dev = "cuda:0"
+    dims, S, nset = O.LLAMA2_7B, args.ctx, 8
+    H, F = dims.hidden, dims.ffn
+    g = torch.Generator().manual_seed(1)
+    sets = []
+    for i in range(nset):
+        w, x, res, k, v, cos, sin = O.make_llama_attn_inputs(dims, S, seed=i)
+        gu = (0.02 * torch.randn(2 * F, H, generator=g)).half().to(dev)
+        dn = (0.02 * torch.randn(H, F, generator=g)).half().to(dev)
+        sets.append(dict(x=x.to(dev), qkv=w["w_qkv"].to(dev), o=w["w_o"].to(dev), k=k.to(dev), v=v.to(dev), r1=w["rms1"].to(dev),
+                         gu=gu, dn=dn, cos=cos.to(dev), sin=sin.to(dev)))
+
+    def layer(a):
+        return cf.llama_decoder_layer_full(a["x"], a["qkv"], a["o"], a["k"], a["v"], a["r1"], a["r1"], a["gu"], a["dn"], dims.eps,
+                                           a["cos"], a["sin"], dims.heads)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for a in sets:
+            layer(a)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = [layer(a) for a in sets]
+    for _ in range(max(1, args.warmup // nset)):
+        graph.replay()
+    torch.cuda.synchronize()
+    reps = max(1, args.steps // nset)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / (reps * nset)
+    nbytes = 2 * (3 * H * H + H * H + 3 * F * H) + 2 * 2 * H + S * 2 * H * 2
+    gbps = nbytes / (us * 1e-6) / 1e9
+    print(json.dumps({
+        "metric": "layer_latency_us", "value": round(us, 2), "unit": "us/layer", "n_gpus": 1, "steps": reps * nset, "warmup": args.warmup,
+        "ms_per_step": round(us * 1e-3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"llama2_7b decoder layer (attention block + SwiGLU MLP block, 3 launches), batch-1 decode, context {S}, "
+                               "graph replay over 8 weight sets", "context": S, "hidden": H, "ffn": F},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "traffic": None, "kernel": "k_fused (attention block) + k_gated_up + k_stage_c", "bytes_per_launch": nbytes,
+                     "launch_us": round(us, 2)},
+        "cpu_baseline": None}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8"])
+    ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8", "llama2_7b_layer"])
     ap.add_argument("--ctx", type=int, default=2048, help="KV-cache rows already filled when the timed region starts")
     ap.add_argument("--mode", default="fused", choices=["fused", "split"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -141,6 +196,10 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
     dev = "cuda:0"
+    if args.model == "llama2_7b_layer":
+        if args.ctx == 2048:
+            args.ctx = 4096          # the context this workload is quoted at
+        return bench_llama_layer(args)
     cfg = pkg.PYTHIA_6B9 if args.model == "pythia_6b9" else pkg.PYTHIA_2B8
     K, W = args.steps, args.warmup
     rows = args.ctx + W + K + 40

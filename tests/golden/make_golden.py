@@ -2,7 +2,7 @@
 
 The reference repository holds no stored expected outputs (its scripts compute them live on a CUDA device),
 so the fixtures are produced by this repository's CPU oracle after it has been pinned against HuggingFace
-GPTNeoXLayer, a brute-force loop and closed forms (tests/test_oracle_pins.py).  Inputs are regenerated from
+GPTNeoXLayer / LlamaAttention, a brute-force loop and closed forms (tests/test_oracle_pins.py).  Inputs are regenerated from
 fixed seeds (oracle.neox_oracle.make_layer_weights / make_layer_inputs); only the expected outputs are
 stored, as float32 in one .npz per case.
 
@@ -33,8 +33,27 @@ def inputs(name):
     return dims, S, w, x, k, v, cos, sin
 
 
+# LLaMA attention block (llama_attention_sglang): dims, cache rows, seed
+LLAMA_CASES = {
+    "llama_h1024_s333": (O.LlamaDims(hidden=1024, heads=8, head_dim=128, ffn=0), 333, 7),
+    "llama2_7b_s1024": (O.LLAMA2_7B, 1024, 8),
+}
+
+
+def llama_inputs(name):
+    dims, S, seed = LLAMA_CASES[name]
+    return (dims,) + tuple(O.make_llama_attn_inputs(dims, S, seed=seed))
+
+
 def main():
     torch.set_num_threads(max(1, os.cpu_count() or 1))
+    for name in LLAMA_CASES:
+        dims, w, x, res, k, v, cos, sin = llama_inputs(name)
+        r = O.llama_attention_sglang(x, res, w, k, v, cos, sin, dims, dtype=torch.float64, round_io=True)
+        out = {n: r[n].to(torch.float32).numpy() for n in ("output", "residual", "k_new", "v_new")}
+        path = os.path.join(HERE, name + ".npz")
+        np.savez_compressed(path, **out)
+        print(name, {n: a.shape for n, a in out.items()}, os.path.getsize(path), "bytes")
     for name in CASES:
         dims, S, w, x, k, v, cos, sin = inputs(name)
         r = O.neox_layer_decode(x, w, k, v, cos, sin, S, dims, dtype=torch.float64, round_io=True)

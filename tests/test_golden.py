@@ -58,3 +58,33 @@ def test_hip_matches_golden(name, op):
     assert_close("output", out, want["output"])
     assert_close("k_new", k_new, want["k_new"])
     assert_close("v_new", v_new, want["v_new"])
+
+
+@pytest.mark.parametrize("name", ["llama_h1024_s333"])
+def test_oracle_reproduces_llama_golden(name):
+    dims, w, x, res, k, v, cos, sin = G.llama_inputs(name)
+    want = load(name)
+    r = O.llama_attention_sglang(x, res, w, k, v, cos, sin, dims, dtype=torch.float32)
+    assert torch.equal(r["residual"].float(), want["residual"])
+    for n in ("output", "k_new", "v_new"):
+        assert float((r[n].float() - want[n]).abs().max()) <= 8e-3, n
+        assert float((r[n].float() - want[n]).abs().mean()) <= 1e-4, n
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["llama_h1024_s333", "llama2_7b_s1024"])
+def test_hip_matches_llama_golden(name):
+    import clusterfusion as cf
+    from tests.test_gpu_layer_parity import assert_close
+    print(f"\ncase golden {name}", flush=True)
+    dims, w, x, res, k, v, cos, sin = G.llama_inputs(name)
+    dev = "cuda:0"
+    res_g = res.to(dev)
+    out, _, k_new, v_new = cf.llama_decoder_layer_sglang(x.to(dev), res_g, w["w_qkv"].to(dev), w["w_o"].to(dev), k.to(dev), v.to(dev),
+                                                         w["rms1"].to(dev), dims.eps, cos.to(dev), sin.to(dev), dims.heads)
+    torch.cuda.synchronize()
+    want = load(name)
+    assert_close("output", out, want["output"])
+    assert_close("k_new", k_new, want["k_new"])
+    assert_close("v_new", v_new, want["v_new"])
+    assert torch.equal(res_g.cpu().float().reshape(-1), want["residual"].reshape(-1))
