@@ -219,7 +219,7 @@ def main():
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         dec.set_state(11, args.ctx)
-        # per-kernel durations with HIP events on the launch stream (eager launches, cold weights)
+        # per-kernel durations with HIP events attached to the layer dispatches (eager launches, cold weights)
         layer_ms, lm_ms = [], []
         for _ in range(3):
             per_layer, lm, _total = dec.profile_step()

@@ -1,6 +1,7 @@
 // Kernels and C-ABI entry points of the GPT-NeoX decode step for MI355X (gfx950).
 // The device building blocks and the design overview live in cfpp_device.hpp.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cmath>
 #include <cstdio>
@@ -563,6 +564,11 @@ int launch_check() {
     return e == hipSuccess ? CFPP_OK : (int)e;
 }
 
+// Set by cfpp_stack_profile_step around a layer launch: the fused kernel is then launched with these events
+// attached to its dispatch (kernel start / kernel end), which is the duration a profiler reports.
+struct KernelEvents { hipEvent_t start, stop; };
+thread_local KernelEvents* tl_kernel_events = nullptr;
+
 // ---- template dispatch ---------------------------------------------------------------------------
 template <int NCH>
 int launch_stage_a_t(const LayerParams& p, int grid, hipStream_t st) {
@@ -581,6 +587,12 @@ int launch_fused_t(const LayerParams& p, int grid, hipStream_t st) {
     static int coop = env_int("CFPP_COOPERATIVE", 0);
     LayerParams pp = p;
     void* args[] = {&pp};
+    if (tl_kernel_events) {
+        // profiling: the events are attached to the dispatch itself and stamp the start and the end of the kernel
+        CFPP_HIP(hipExtLaunchKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st, tl_kernel_events->start,
+                                    tl_kernel_events->stop, 0));
+        return CFPP_OK;
+    }
     if (coop) CFPP_HIP(hipLaunchCooperativeKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st));
     else CFPP_HIP(hipLaunchKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st));
     return CFPP_OK;
@@ -1213,6 +1225,14 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
     const int L = s->desc.n_layers;
     std::vector<hipEvent_t> ev(L + 3);
     for (auto& e : ev) CFPP_HIP(hipEventCreate(&e));
+    // fused mode: one kernel per layer, timed from its own start to its own end; split mode (three kernels per layer):
+    // stream events between the layers, which include the launch gaps
+    const bool fused = s->desc.mode == CFPP_MODE_FUSED && s->desc.dims.heads <= fused_grid() * kStreamers;
+    std::vector<KernelEvents> kev(fused ? L : 0);
+    for (auto& k : kev) {
+        CFPP_HIP(hipEventCreate(&k.start));
+        CFPP_HIP(hipEventCreate(&k.stop));
+    }
     int rc = CFPP_OK;
     {
         const cfpp_neox_dims& d = s->desc.dims;
@@ -1223,7 +1243,9 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
         rc = launch_check();
         for (int l = 0; l < L && !rc; ++l) {
             CFPP_HIP(hipEventRecord(ev[l], st));
+            if (fused) tl_kernel_events = &kev[l];
             rc = stack_enqueue_layer(s, l, st);
+            tl_kernel_events = nullptr;
         }
         if (!rc) {
             CFPP_HIP(hipEventRecord(ev[L], st));
@@ -1241,7 +1263,8 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
     if (!rc) {
         for (int l = 0; l < L; ++l) {
             float ms = 0.f;
-            CFPP_HIP(hipEventElapsedTime(&ms, ev[l], ev[l + 1]));
+            if (fused) CFPP_HIP(hipEventElapsedTime(&ms, kev[l].start, kev[l].stop));
+            else CFPP_HIP(hipEventElapsedTime(&ms, ev[l], ev[l + 1]));
             if (layer_ms) layer_ms[l] = ms;
         }
         float ms = 0.f;
@@ -1251,6 +1274,7 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
         if (total_ms) *total_ms = ms;
     }
     for (auto& e : ev) (void)hipEventDestroy(e);
+    for (auto& k : kev) { (void)hipEventDestroy(k.start); (void)hipEventDestroy(k.stop); }
     (void)hipEventDestroy(end);
     return rc;
 }
