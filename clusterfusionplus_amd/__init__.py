@@ -35,6 +35,8 @@ if not _missing:
     __all__ = [n for n in dir(_native) if not n.startswith("_")]
     globals().update({n: getattr(_native, n) for n in __all__})
 
-    from .model import NeoxConfig, PYTHIA_2B8, PYTHIA_6B9, NeoxDecoder, layer_tensor_order, rope_tables  # noqa: E402
+    from .model import (NeoxConfig, PYTHIA_2B8, PYTHIA_6B9, NeoxDecoder, layer_tensor_order, rope_tables,  # noqa: E402
+                        layer_tensors_from_hf, kv_cache_from_hf)
 
-    __all__ += ["NeoxConfig", "PYTHIA_2B8", "PYTHIA_6B9", "NeoxDecoder", "layer_tensor_order", "rope_tables"]
+    __all__ += ["NeoxConfig", "PYTHIA_2B8", "PYTHIA_6B9", "NeoxDecoder", "layer_tensor_order", "rope_tables",
+                "layer_tensors_from_hf", "kv_cache_from_hf"]

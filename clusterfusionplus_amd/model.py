@@ -41,6 +41,45 @@ def rope_tables(positions: int, rotary_dim: int, base: float = 10000.0, device="
     return emb.cos().float().to(device).contiguous(), emb.sin().float().to(device).contiguous()
 
 
+# ---- prefill -> decode hand-off: HuggingFace GPT-NeoX modules and caches to this library's layout -------------
+
+def layer_tensors_from_hf(hf_layer, dtype=torch.float16, device=None) -> Dict[str, torch.Tensor]:
+    """The 12 per-layer tensors of a HuggingFace `GPTNeoXLayer`, keyed by `layer_tensor_order`
+    (the set reference tests/benchmark_decode.py:83-96 pulls out of the module).  HF keeps `query_key_value`
+    head-interleaved `[head][q|k|v][D]`, which is the layout the kernels read, so nothing is re-ordered."""
+    a, m = hf_layer.attention, hf_layer.mlp
+    src = {
+        "ln_w": hf_layer.input_layernorm.weight, "ln_b": hf_layer.input_layernorm.bias,
+        "w_qkv": a.query_key_value.weight, "b_qkv": a.query_key_value.bias,
+        "w_o": a.dense.weight, "b_o": a.dense.bias,
+        "post_ln_w": hf_layer.post_attention_layernorm.weight, "post_ln_b": hf_layer.post_attention_layernorm.bias,
+        "w_up": m.dense_h_to_4h.weight, "b_up": m.dense_h_to_4h.bias,
+        "w_down": m.dense_4h_to_h.weight, "b_down": m.dense_4h_to_h.bias,
+    }
+    out = {}
+    for k in layer_tensor_order:
+        t = src[k].detach().to(dtype)
+        out[k] = (t.to(device) if device is not None else t).contiguous()
+    return out
+
+
+def kv_cache_from_hf(key: torch.Tensor, value: torch.Tensor, rows: int, dtype=torch.float16, device=None):
+    """HF `past_key_values` of one layer, `[1, heads, S, D]` each, to the `[rows, heads*D]` caches the decode step
+    reads and appends to (`permute(0,2,1,3).reshape(S, H)`, reference tests/benchmark_decode.py:99-108).
+    Returns (k_cache, v_cache, S); rows >= S + the tokens to be generated."""
+    if key.dim() != 4 or key.shape[0] != 1 or key.shape != value.shape:
+        raise ValueError(f"expected key/value of shape [1, heads, S, D], got {tuple(key.shape)} / {tuple(value.shape)}")
+    _, nh, S, D = key.shape
+    if rows < S:
+        raise ValueError(f"rows ({rows}) < cached positions ({S})")
+    dev = device if device is not None else key.device
+    kc = torch.zeros((rows, nh * D), dtype=dtype, device=dev)
+    vc = torch.zeros((rows, nh * D), dtype=dtype, device=dev)
+    kc[:S] = key.detach().permute(0, 2, 1, 3).reshape(S, nh * D).to(device=dev, dtype=dtype)
+    vc[:S] = value.detach().permute(0, 2, 1, 3).reshape(S, nh * D).to(device=dev, dtype=dtype)
+    return kc, vc, S
+
+
 class NeoxDecoder:
     """Greedy batch-1 decoder over device-resident weights and KV caches.
 

@@ -100,3 +100,38 @@ def test_rope_tables_match_oracle():
     c, s = rope_tables(300, 20, device="cpu")
     c2, s2 = rope_table(torch.arange(300), 20)
     assert torch.equal(c, c2) and torch.equal(s, s2)
+
+
+def test_hf_hand_off_helpers_reproduce_the_hf_layer():
+    """layer_tensors_from_hf / kv_cache_from_hf: a prefill done by HuggingFace, one decode step by the oracle on the
+    converted tensors == the HF layer's own decode step."""
+    pytest.importorskip("transformers")
+    import torch
+    from transformers import DynamicCache
+    from clusterfusionplus_amd.model import kv_cache_from_hf, layer_tensors_from_hf, layer_tensor_order
+    from oracle import hf_neox, neox_oracle as O
+    dims = O.NeoxDims(hidden=64, heads=4, head_dim=16, rotary_dim=4, ffn=256)
+    w0 = O.make_layer_weights(dims, layer=3, w_std=0.2, b_std=0.1)
+    layer = hf_neox.build_hf_layer(dims, w0, dtype=torch.float64)
+    w = layer_tensors_from_hf(layer, dtype=torch.float64)
+    assert tuple(w) == layer_tensor_order
+    for k in layer_tensor_order:
+        assert torch.equal(w[k].reshape(-1), w0[k].double().reshape(-1)), k
+    S = 6
+    g = torch.Generator().manual_seed(4)
+    key = torch.randn(1, dims.heads, S, dims.head_dim, generator=g, dtype=torch.float64)
+    val = torch.randn(1, dims.heads, S, dims.head_dim, generator=g, dtype=torch.float64)
+    kc, vc, n = kv_cache_from_hf(key, val, rows=S + 2, dtype=torch.float64)
+    assert n == S and kc.shape == (S + 2, dims.hidden) and torch.equal(kc[S:], torch.zeros(2, dims.hidden, dtype=torch.float64))
+    x = torch.randn(1, dims.hidden, generator=g, dtype=torch.float64)
+    cos, sin = O.rope_table(torch.tensor([S]), dims.rotary_dim)
+    got = O.neox_layer_decode(x, w, kc, vc, cos, sin, S, dims, dtype=torch.float64, round_io=False)
+    cache = DynamicCache(ddp_cache_data=[(key.clone(), val.clone())])
+    c = cos.double().reshape(-1)[: dims.rotary_dim][None, None]
+    s_ = sin.double().reshape(-1)[: dims.rotary_dim][None, None]
+    with torch.no_grad():
+        want = layer(x.reshape(1, 1, -1), attention_mask=None, layer_past=cache, position_embeddings=(c, s_))
+    want = want[0] if isinstance(want, tuple) else want
+    assert torch.allclose(got["output"], want.reshape(1, -1), atol=1e-6, rtol=0)
+    with pytest.raises(ValueError):
+        kv_cache_from_hf(key, val, rows=S - 1)
