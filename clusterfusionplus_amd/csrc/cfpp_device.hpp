@@ -887,8 +887,8 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     last = first_lane(last);
     if (last) {
         // The last wave of this head merges the splits.  Lane i fetches (m_i, l_i) of split i, so the
-        // scales come from one round trip; the accumulators (two dims per lane) are fetched 16
-        // splits at a time and added in split order.
+        // scales come from one round trip; the accumulators (two dims per lane) are fetched kMergeBatch
+        // splits at a time, together with the scales, and added in split order.
         const size_t hb = (size_t)head * kMaxSplit;
         float mi = kNegBig, li = 0.f;
         if (lane < nsplit) ld_agent2(p.part_ml + (hb + lane) * 2, mi, li);

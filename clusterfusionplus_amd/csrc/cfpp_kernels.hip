@@ -209,18 +209,20 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
 }
 
 // ---- fused mode: one persistent launch ---------------------------------------------------------
-// One workgroup per compute unit, eight waves: four streaming waves (one per SIMD) and four helper waves.
-//   streaming wave: first QKV tile in flight -> LayerNorm -> its QKV rows -> bump kBarQkv -> its MLP-up
-//                   rows, phase by phase, bumping kBarUp + g after phase g -> (helps with attention items
-//                   if any are left) -> MLP-down rows of stage C, phase by phase (first weight tile in
-//                   flight, then wait for kBarUp + g): the first down phase only needs the first up phase
-//                   of every workgroup, so a workgroup that is late with its MLP-up rows holds up nobody
-//                   until the second half of the down pass.
-//   helper wave:    waits for kBarQkv, then takes (head, split) attention items from the workgroup's
-//                   queue at raised wave priority, then does the O-projection rows of stage C (first
-//                   rows in flight, then wait for kBarHeads).  Attention is a chain of dependent memory
-//                   round trips; it and the O projection run beside the MLP-up / MLP-down streaming
-//                   instead of in front of it.
+// One workgroup per compute unit, eight waves: four streaming waves (one per SIMD) and four attention waves.
+//   all waves:      LayerNorm shared through LDS (each wave loads one 512-half chunk of the row).
+//   streaming wave: first QKV tile requested before the LayerNorm -> its QKV rows -> bump kBarQkv -> its MLP-up
+//                   tiles, phase by phase (by ticket within a team of workgroups when the phases are long
+//                   enough), bumping kBarUp + g after phase g -> MLP-down rows of stage C, phase by phase
+//                   (first weight tile in flight, then wait for kBarUp + g): the first down phase only needs
+//                   the first up phase of every workgroup, so a workgroup that is late with its MLP-up rows
+//                   holds up nobody until the second half of the down pass.
+//   attention wave: owns one (head, split) item: requests its first K/V tiles and RoPE coefficients, waits for
+//                   kBarQkv, runs the item at raised wave priority (the last wave of a head merges its
+//                   splits and bumps kBarHeads), then does the O-projection rows of stage C (all rows
+//                   requested, then wait for kBarHeads).  Attention is a chain of dependent memory round
+//                   trips; it and the O projection run beside the MLP-up / MLP-down streaming instead of in
+//                   front of it.
 //   all waves:      row reduction in LDS, bias, residual.
 // Nothing is reset at the end: counters zero themselves and flags carry a launch generation.  All workgroups must be
 // co-resident (the host launches one per compute unit); every wait is bounded.
