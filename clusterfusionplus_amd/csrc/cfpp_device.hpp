@@ -69,6 +69,7 @@ struct LayerParams {
     const int* d_seq_len;
     int max_split;      // cap on the KV splits per head (<= kMaxSplit)
     int row_walk_strided;   // streaming waves take interleaved instead of contiguous row ranges
+    int arrival_agents;     // an idle attention wave carries the streaming waves' MLP-up arrivals to the device-wide counters
     int dyn_up;             // MLP-up tiles handed out dynamically within teams of workgroups: 1 yes, 0 no, -1 by size
     // layer family switches (defaults = GPT-NeoX): RMSNorm instead of LayerNorm; where head h's raw q, k, v sit in
     // qkv_raw (NeoX interleaves [h][q|k|v][D]: stride 3D, offsets D and 2D; LLaMA stacks [q;k;v]: stride D,

@@ -276,6 +276,32 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
     const int nitems = p.heads * nsplit;
     const int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
     trace_mark(p, 1);
+    // Counting an arrival device-wide is two dependent atomic round trips for the wave that does it, and a
+    // streaming wave that stops for them falls behind its workgroup (and then is the last one again at the next
+    // event).  When the workgroup has an attention wave without an item (fewer than four items), the streaming
+    // waves only drain their stores and count themselves in LDS at the MLP-up events, and that idle wave carries
+    // the count to the device-wide counters.  (Not at the QKV event: the attention waves wait for that one, and
+    // an arrival that goes through another wave reaches them later.)
+    const bool agent_up = p.arrival_agents && attn_count < kStreamers;
+    auto stream_arrive = [&](int event, int* lds_ctr, bool agent) {
+        if (agent) {
+            drain_memory_ops();
+            if (lane == 0) __hip_atomic_fetch_add(lds_ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        } else {
+            event_arrive(p.bar, p.grp, p.mbox, event, G, lds_ctr, kStreamers, tag);
+        }
+    };
+    auto agent_serve = [&](int event, int* lds_ctr) {
+        if (lane == 0) {
+            int spins = 0;
+            while (__hip_atomic_load(lds_ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < kStreamers) {
+                __builtin_amdgcn_s_sleep(1);
+                if (++spins > kSpinLimit * 8) { raise_status(status, kStatusSpin); break; }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        event_arrive(p.bar, p.grp, p.mbox, event, G, nullptr, 1, tag);
+    };
 
     if (wave < kStreamers) {
         RowPark spark{park_mem[wave], 0};
@@ -302,7 +328,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
                     utm = make_team<kUpRpi>(p, 2 + g, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F), b, G, wave);
                     team_prefetch<NCH, kUpRpi, EX>(p.w_up, p.H, utm, lane, ut);
                 }
-                event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &q.arrived[1 + g], kStreamers, tag);
+                stream_arrive(kBarUp + g, &q.arrived[1 + g], agent_up);
                 trace_mark(p, g == kUpPhases - 1 ? 5 : 12);
             }
         } else {
@@ -319,7 +345,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
                     uw = row_walk<kUpRpi>(false, b * kStreamers + wave, nsw, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F));
                     up_prefetch<NCH, EX>(p, uw, lane, u0);
                 }
-                event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &q.arrived[1 + g], kStreamers, tag);
+                stream_arrive(kBarUp + g, &q.arrived[1 + g], agent_up);
                 trace_mark(p, g == kUpPhases - 1 ? 5 : 12);
             }
         }
@@ -335,8 +361,11 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
             trace_mark(p, 3);
             attention_item(p, it, lane, G, tag);
             trace_mark(p, 4);
+            __builtin_amdgcn_s_setprio(0);
+        } else if (hw == kStreamers - 1 && agent_up) {
+#pragma unroll
+            for (int g = 0; g < kUpPhases; ++g) agent_serve(kBarUp + g, &q.arrived[1 + g]);
         }
-        __builtin_amdgcn_s_setprio(0);
     }
     trace_mark(p, 9);
     {
@@ -717,6 +746,7 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     p.norm_rms = 0; p.qkv_head_stride = 3 * d->head_dim; p.qkv_k_off = d->head_dim; p.qkv_v_off = 2 * d->head_dim;
     p.append_kv = 1; p.x_add = nullptr; p.x_sum_out = nullptr; p.c_add_sum = 0;
     p.dyn_up = env_int("CFPP_DYN_UP", -1);
+    p.arrival_agents = env_int("CFPP_ARRIVAL_AGENTS", 1);
     char* ws = reinterpret_cast<char*>(workspace);
     p.qkv_raw = reinterpret_cast<float*>(ws + L.qkv_raw);
     p.attn_vec = reinterpret_cast<half_t*>(ws + L.attn_vec);
