@@ -69,6 +69,7 @@ struct LayerParams {
     const int* d_seq_len;
     int max_split;      // cap on the KV splits per head (<= kMaxSplit)
     int row_walk_strided;   // streaming waves take interleaved instead of contiguous row ranges
+    const int* kv_rows;     // paged caches: cache row r of this sequence lives in row kv_rows[r] of k_cache / v_cache (null: r itself)
     int arrival_agents;     // an idle attention wave carries the streaming waves' MLP-up arrivals to the device-wide counters
     int dyn_up;             // MLP-up tiles handed out dynamically within teams of workgroups: 1 yes, 0 no, -1 by size
     // layer family switches (defaults = GPT-NeoX): RMSNorm instead of LayerNorm; where head h's raw q, k, v sit in
@@ -745,6 +746,8 @@ struct AttnItem {
     RopeCoeffs rc;
 };
 // tile i of the item; rows past the end re-read the last row (masked when used): no conditional loads
+// PAGED: rows go through p.kv_rows
+template <bool PAGED = false>
 __device__ __forceinline__ void attn_load_tile(const LayerParams& p, const AttnItem& it, KvTile& kv, int i, int lane) {
     const int grp = lane >> 4, sub = lane & 15;
     const int d0 = sub * 8 < p.D ? sub * 8 : 0;      // idle lanes read (and ignore) the first dims
@@ -753,19 +756,21 @@ __device__ __forceinline__ void attn_load_tile(const LayerParams& p, const AttnI
     const int r = it.begin + i * kAttnTileRows + grp;
 #pragma unroll
     for (int t = 0; t < kAttnT; ++t) {
-        const int row = (r + t * 4 < it.end) ? r + t * 4 : it.end - 1;
+        int row = (r + t * 4 < it.end) ? r + t * 4 : it.end - 1;
+        if (PAGED) row = p.kv_rows[row];
         kv.k[t] = ld16(kc + (size_t)row * p.H);
         kv.v[t] = ld16(vc + (size_t)row * p.H);
     }
 }
+template <bool PAGED = false>
 __device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it, int head, int sp, int nsplit, int S, int lane) {
     it.head = head; it.sp = sp; it.nsplit = nsplit; it.S = S;
     const int chunk = (S + nsplit - 1) / nsplit;
     it.begin = sp * chunk;
     it.end = (it.begin + chunk < S) ? it.begin + chunk : S;
     it.ntiles = it.begin < it.end ? (it.end - it.begin + kAttnTileRows - 1) / kAttnTileRows : 0;
-    if (it.ntiles > 0) attn_load_tile(p, it, it.t0, 0, lane);
-    if (it.ntiles > 1) attn_load_tile(p, it, it.t1, 1, lane);
+    if (it.ntiles > 0) attn_load_tile<PAGED>(p, it, it.t0, 0, lane);
+    if (it.ntiles > 1) attn_load_tile<PAGED>(p, it, it.t1, 1, lane);
     const int sub = lane & 15;
     const bool act = sub * 8 < p.D;
     const float* __restrict__ cs = p.cos + (size_t)S * p.rope_stride;   // stride 0: the row is the position
@@ -774,6 +779,7 @@ __device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it
 }
 
 // nwg_to_signal > 0 (fused kernel): a completed head counts towards the kBarHeads event of that many workgroups.
+template <bool PAGED = false>
 __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& it, int lane, int nwg_to_signal, int tag) {
     const int grp = lane >> 4, sub = lane & 15;
     const int D = p.D, H = p.H;
@@ -803,7 +809,13 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
             const size_t o = (size_t)head * D + d0;
             *reinterpret_cast<u32x4*>(p.k_new + o) = kp;
             *reinterpret_cast<u32x4*>(p.v_new + o) = vp;
-            if (p.append_kv && S < p.cache_rows) {
+            if (PAGED) {
+                if (p.append_kv) {
+                    const size_t slot = (size_t)p.kv_rows[S];
+                    *reinterpret_cast<u32x4*>(p.k_cache + slot * H + o) = kp;
+                    *reinterpret_cast<u32x4*>(p.v_cache + slot * H + o) = vp;
+                }
+            } else if (p.append_kv && S < p.cache_rows) {
                 *reinterpret_cast<u32x4*>(p.k_cache + (size_t)S * H + o) = kp;
                 *reinterpret_cast<u32x4*>(p.v_cache + (size_t)S * H + o) = vp;
             }
@@ -848,12 +860,12 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     };
     if (it.ntiles > 0) process(it.t0, 0);
     __builtin_amdgcn_sched_barrier(0);
-    if (it.ntiles > 2) attn_load_tile(p, it, it.t0, 2, lane);     // the third tile travels while the second is reduced
+    if (it.ntiles > 2) attn_load_tile<PAGED>(p, it, it.t0, 2, lane);     // the third tile travels while the second is reduced
     __builtin_amdgcn_sched_barrier(0);
     if (it.ntiles > 1) process(it.t1, 1);
     __builtin_amdgcn_sched_barrier(0);
     for (int i = 2; i < it.ntiles; ++i) {
-        if (i != 2) attn_load_tile(p, it, it.t0, i, lane);
+        if (i != 2) attn_load_tile<PAGED>(p, it, it.t0, i, lane);
         process(it.t0, i);
     }
 

@@ -507,6 +507,176 @@ __global__ void k_fill_zero(uint32_t* p, size_t n) {
 // =================================================================================================
 namespace {
 
+// ---- batched decode over paged caches ---------------------------------------------------------------------
+// Several sequences take one decode step together (reference include/5090/llama/kernel_batch_sglang.cuh:43-60: one
+// cluster per (sequence, head)).  Here the weight rows are streamed once for a group of up to kBatchTile
+// sequences: the normalised input rows of the group sit in LDS as fp16, and every weight tile in registers is
+// multiplied with each of them before the next tile arrives.  Three launches: norm + QKV rows (k_batch_gemv),
+// attention items over (sequence, head, split) with cache rows looked up through the page table
+// (k_batch_attn), O-projection rows (k_batch_gemv again).
+constexpr int kBatchTile = 8;        // sequences sharing one pass over the weights
+constexpr int kBatchParkRows = 32;   // rows a wave may own in one launch
+struct BatchGemv {
+    const half_t* W; int R, K;                    // weight rows [R, K]
+    const half_t *x, *x_add; half_t* sum_out;     // [batch][K]; x_add: optional second row, sum_out: fp16(x + x_add)
+    const half_t* norm_w; float eps;              // RMSNorm weight (null: the rows are used as they are)
+    float* out_f32; half_t* out_f16;              // [batch][R], one of the two
+    int batch;
+};
+template <int NCH, bool EX>
+__global__ __launch_bounds__(kStreamers * 64) void k_batch_gemv(BatchGemv a) {
+    __shared__ __attribute__((aligned(16))) half_t xs[kBatchTile][NCH * kChunk];
+    __shared__ float park[kStreamers][kBatchParkRows * kBatchTile];
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int gw = blockIdx.x * kStreamers + wave, nw = gridDim.x * kStreamers;
+    constexpr int RPI = 2;
+    const RowWalk rw = row_walk<RPI>(false, gw, nw, 0, a.R);
+    const int nrows = rw.end > rw.first ? rw.end - rw.first : 0;
+    for (int t0 = 0; t0 < a.batch; t0 += kBatchTile) {
+        const int nb = a.batch - t0 < kBatchTile ? a.batch - t0 : kBatchTile;
+        __syncthreads();     // the previous group's rows in LDS are no longer needed
+        RowTile<NCH, RPI> ta, tb;
+        if (rw.ntiles > 0) load_row_tile<NCH, RPI, EX>(ta, a.W, a.K, rw.first, 1, rw.end, lane);
+        // a wave prepares whole rows: sum with the residual (rounded to fp16), RMS statistics in fp32, fp16 result
+        for (int tk = wave; tk < nb; tk += kStreamers) {
+            const size_t base = (size_t)(t0 + tk) * a.K;
+            float v[NCH][8];
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                const int col = i * kChunk + lane * 8;
+                const bool in = col < a.K;
+                u32x4 r = {0u, 0u, 0u, 0u};
+                if (in) r = ld16(a.x + base + col);
+                unpack8(r, v[i]);
+                if (a.x_add != nullptr) {
+                    u32x4 ra = {0u, 0u, 0u, 0u};
+                    if (in) ra = ld16(a.x_add + base + col);
+                    float w[8];
+                    unpack8(ra, w);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[i][j] += w[j];
+                    r = pack8(v[i]);
+                    unpack8(r, v[i]);
+                    if (in && a.sum_out != nullptr && blockIdx.x == 0) *reinterpret_cast<u32x4*>(a.sum_out + base + col) = r;
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ss += v[i][j] * v[i][j];
+            }
+            float rstd = 1.f;
+            if (a.norm_w != nullptr) rstd = 1.0f / sqrtf(wave_sum(ss) / (float)a.K + a.eps);
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                const int col = i * kChunk + lane * 8;
+                if (a.norm_w != nullptr) {
+                    float g[8];
+                    u32x4 rg = {0u, 0u, 0u, 0u};
+                    if (col < a.K) rg = ld16(a.norm_w + col);
+                    unpack8(rg, g);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[i][j] = v[i][j] * rstd * g[j];
+                }
+                *reinterpret_cast<u32x4*>(&xs[tk][col]) = pack8(v[i]);
+            }
+        }
+        __syncthreads();
+        int prow = 0;
+        auto consume = [&](const RowTile<NCH, RPI>& t, int valid) {
+            for (int tk = 0; tk < nb; ++tk) {
+                half2_t xv[NCH][4];
+#pragma unroll
+                for (int i = 0; i < NCH; ++i) {
+                    const u32x4 q = *reinterpret_cast<const u32x4*>(&xs[tk][i * kChunk + lane * 8]);
+                    xv[i][0] = as_h2(q.x); xv[i][1] = as_h2(q.y); xv[i][2] = as_h2(q.z); xv[i][3] = as_h2(q.w);
+                }
+#pragma unroll
+                for (int j = 0; j < RPI; ++j) {
+                    float acc = 0.f;
+#pragma unroll
+                    for (int i = 0; i < NCH; ++i) acc = dot8(t.w[j][i], xv[i], acc);
+                    acc = wave_sum(acc);
+                    if (j < valid && lane == 0) park[wave][tk * kBatchParkRows + prow + j] = acc;
+                }
+            }
+            prow += valid;
+        };
+        auto valid_rows = [&](int t) { const int left = nrows - t * RPI; return left < RPI ? left : RPI; };
+        auto load = [&](RowTile<NCH, RPI>& t, int i) { load_row_tile<NCH, RPI, EX>(t, a.W, a.K, rw.first + i * RPI, 1, rw.end, lane); };
+        int t = 0;
+        for (; t + 2 < rw.ntiles; t += 2) {
+            load(tb, t + 1);
+            consume(ta, RPI);
+            __builtin_amdgcn_sched_barrier(0);
+            load(ta, t + 2);
+            consume(tb, RPI);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (t + 1 < rw.ntiles) {
+            load(tb, t + 1);
+            consume(ta, RPI);
+            __builtin_amdgcn_sched_barrier(0);
+            consume(tb, valid_rows(t + 1));
+        } else if (t < rw.ntiles) {
+            consume(ta, valid_rows(t));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // one (sequence, row) result per lane
+        for (int idx = lane; idx < nrows * nb; idx += kWave) {
+            const int tk = idx / nrows, r = idx - tk * nrows;
+            const float val = park[wave][tk * kBatchParkRows + r];
+            const size_t o = (size_t)(t0 + tk) * a.R + rw.first + r;
+            if (a.out_f32 != nullptr) a.out_f32[o] = val;
+            else a.out_f16[o] = (half_t)val;
+        }
+    }
+}
+
+struct BatchAttn {
+    int batch, layer_id;
+    const int *indptr, *indices;                           // page table: rows indices[indptr[b] .. indptr[b+1]-1) hold
+                                                           // the sequence, the last entry is the row of the new token
+    const unsigned long long *k_ptrs, *v_ptrs;             // per-layer cache base addresses
+    const long long* positions;                            // [batch]
+    const float* cos_sin;                                  // [positions][D]: cos of the D/2 pair angles, then sin
+};
+// One wave per (sequence, head, split); the parameter block of the single-sequence kernels, re-pointed at the
+// sequence's rows.
+__global__ __launch_bounds__(kStreamers * 64) void k_batch_attn(LayerParams p, BatchAttn b) {
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int item = blockIdx.x * kStreamers + wave;
+    const int per_seq = p.heads * p.max_split;
+    const int seq = item / per_seq;
+    if (seq >= b.batch) return;
+    const int rem = item - seq * per_seq;
+    const int head = rem / p.max_split, sp = rem - head * p.max_split;
+    const int start = b.indptr[seq];
+    int S = b.indptr[seq + 1] - 1 - start;
+    if (S < 0) {
+        if (lane == 0) raise_status(p.bar + kBarStatus, kStatusSeq);
+        return;
+    }
+    const int nsplit = effective_split(p, S);
+    if (sp >= nsplit) return;
+    LayerParams q = p;
+    q.kv_rows = b.indices + start;
+    q.k_cache = reinterpret_cast<half_t*>(b.k_ptrs[b.layer_id]);
+    q.v_cache = reinterpret_cast<half_t*>(b.v_ptrs[b.layer_id]);
+    q.cos = b.cos_sin + (size_t)b.positions[seq] * p.D;
+    q.sin = q.cos + p.D / 2;
+    q.rope_stride = 0;
+    q.qkv_raw += (size_t)seq * 3 * p.H;
+    q.attn_vec += (size_t)seq * p.H;
+    q.k_new += (size_t)seq * p.H;
+    q.v_new += (size_t)seq * p.H;
+    q.part_ml += (size_t)seq * p.heads * kMaxSplit * 2;
+    q.part_acc += (size_t)seq * p.heads * kMaxSplit * p.D;
+    q.head_cnt += (size_t)seq * p.heads;
+    AttnItem it;
+    attn_prefetch<true>(q, it, head, sp, nsplit, S, lane);
+    attention_item<true>(q, it, lane, 0, 0);
+}
+
+
 struct DeviceInfo {
     int cus = 0;
     bool ok = false;
@@ -785,6 +955,44 @@ int run_split(const Plan& pl, LayerParams& p, int seq_hint, hipStream_t st) {
 // =================================================================================================
 // C ABI
 // =================================================================================================
+// ---- launchers of the batched LLaMA attention block ---------------------------------------------------
+namespace {
+struct BatchLayout { size_t qkv_raw, attn_vec, k_new, v_new, part_ml, part_acc, head_cnt, bar, total; };
+BatchLayout batch_layout(const cfpp_neox_dims& d, int batch) {
+    BatchLayout w{};
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t at = off; off += align_up(bytes, 256); return at; };
+    const size_t B = (size_t)batch, H = (size_t)d.hidden;
+    w.qkv_raw = take(B * 3 * H * 4);
+    w.attn_vec = take(B * H * 2);
+    w.k_new = take(B * H * 2);
+    w.v_new = take(B * H * 2);
+    w.part_ml = take(B * d.heads * kMaxSplit * 2 * 4);
+    w.part_acc = take(B * d.heads * kMaxSplit * (size_t)d.head_dim * 4);
+    w.head_cnt = take(B * d.heads * 4);
+    w.bar = take(64 * 4);
+    w.total = off;
+    return w;
+}
+template <int NCH>
+int launch_batch_gemv_t(const BatchGemv& a, int grid, hipStream_t st) {
+    if (a.K == NCH * kChunk) hipLaunchKernelGGL((k_batch_gemv<NCH, true>), dim3(grid), dim3(kStreamers * 64), 0, st, a);
+    else hipLaunchKernelGGL((k_batch_gemv<NCH, false>), dim3(grid), dim3(kStreamers * 64), 0, st, a);
+    return (int)hipGetLastError();
+}
+int launch_batch_gemv(int nch, const BatchGemv& a, int grid, hipStream_t st) {
+    switch (nch) {
+        case 1: return launch_batch_gemv_t<1>(a, grid, st);
+        case 2: return launch_batch_gemv_t<2>(a, grid, st);
+        case 4: return launch_batch_gemv_t<4>(a, grid, st);
+        case 5: return launch_batch_gemv_t<5>(a, grid, st);
+        case 8: return launch_batch_gemv_t<8>(a, grid, st);
+        default: return CFPP_ERR_DIMS;
+    }
+}
+}  // namespace
+
+
 extern "C" {
 
 const char* cfpp_version(void) { return "cfpp 0.1 (gfx950)"; }
@@ -800,6 +1008,7 @@ const char* cfpp_status_str(int s) {
         case CFPP_ERR_MODE: return "unknown mode";
         case CFPP_ERR_DEVICE: return "device-side failure flag raised";
         case CFPP_ERR_ALIGN: return "tensor pointer is not 16-byte aligned";
+        case CFPP_ERR_ALIAS: return "an output overlaps an input";
         default: break;
     }
     if (s > 0) return hipGetErrorString((hipError_t)s);
@@ -925,6 +1134,84 @@ int cfpp_llama_mlp(const cfpp_llama_mlp_args* m, void* workspace, size_t workspa
     int rc = launch_gated_up(pl, p, grid, st);
     if (rc) return rc;
     return launch_stage_c(pl, p, grid, st);
+}
+
+// ---- LLaMA attention block, batched over paged caches ---------------------------------------------------
+size_t cfpp_llama_batch_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim, int32_t batch) {
+    const cfpp_neox_dims d = llama_dims(hidden, heads, head_dim, 1e-6f);
+    if (check_dims(&d) || batch < 1) return 0;
+    return batch_layout(d, batch).total;
+}
+
+int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!a || !workspace) return CFPP_ERR_NULL;
+    const cfpp_neox_dims d = llama_dims(a->hidden, a->heads, a->head_dim, a->eps);
+    int rc = check_dims(&d);
+    if (rc) return rc;
+    if (a->batch < 1 || a->layer_id < 0) return CFPP_ERR_DIMS;
+    const void* req[] = {a->rms_w, a->w_qkv, a->w_o, a->input, a->residual, a->residual_out, a->output, a->cos_sin};
+    for (const void* q : req) {
+        if (!q) return CFPP_ERR_NULL;
+        if (!aligned16(q)) return CFPP_ERR_ALIGN;
+    }
+    if (!a->paged_kv_indptr || !a->paged_kv_indices || !a->k_cache_ptrs || !a->v_cache_ptrs || !a->positions) return CFPP_ERR_NULL;
+    // the sum input + residual is written while other workgroups still read both rows
+    if (a->residual_out == a->input || a->residual_out == a->residual) return CFPP_ERR_ALIAS;
+    const BatchLayout L = batch_layout(d, a->batch);
+    if (workspace_bytes < L.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CFPP_ERR_WORKSPACE;
+    const int nch = (d.hidden + kChunk - 1) / kChunk;
+    const int grid = streaming_grid();
+    const int waves = grid * kStreamers;
+    if ((3 * d.hidden + waves - 1) / waves + 2 > kBatchParkRows) return CFPP_ERR_DIMS;
+    char* ws = reinterpret_cast<char*>(workspace);
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    auto h = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
+
+    BatchGemv g{};
+    g.W = h(a->w_qkv); g.R = 3 * d.hidden; g.K = d.hidden;
+    g.x = h(a->input); g.x_add = h(a->residual); g.sum_out = reinterpret_cast<half_t*>(a->residual_out);
+    g.norm_w = h(a->rms_w); g.eps = a->eps;
+    g.out_f32 = reinterpret_cast<float*>(ws + L.qkv_raw); g.out_f16 = nullptr;
+    g.batch = a->batch;
+    if ((rc = launch_batch_gemv(nch, g, grid, st))) return rc;
+
+    LayerParams p{};
+    p.H = d.hidden; p.heads = d.heads; p.D = d.head_dim; p.rot = d.head_dim; p.F = 0;
+    p.eps = a->eps;
+    p.qscale = (float)(1.4426950408889634 / std::sqrt((double)d.head_dim));
+    p.qkv_raw = reinterpret_cast<float*>(ws + L.qkv_raw);
+    p.attn_vec = reinterpret_cast<half_t*>(ws + L.attn_vec);
+    p.k_new = reinterpret_cast<half_t*>(ws + L.k_new);
+    p.v_new = reinterpret_cast<half_t*>(ws + L.v_new);
+    p.part_ml = reinterpret_cast<float*>(ws + L.part_ml);
+    p.part_acc = reinterpret_cast<float*>(ws + L.part_acc);
+    p.head_cnt = reinterpret_cast<int*>(ws + L.head_cnt);
+    p.bar = reinterpret_cast<int*>(ws + L.bar);
+    p.qkv_head_stride = d.head_dim; p.qkv_k_off = d.hidden; p.qkv_v_off = 2 * d.hidden;
+    p.append_kv = 1;
+    // enough (sequence, head, split) items to fill the attention waves about twice, and no more
+    int ms = (2 * waves) / (a->batch * d.heads);
+    ms = ms < 1 ? 1 : (ms > 32 ? 32 : ms);
+    p.max_split = env_int("CFPP_MAX_SPLIT", ms);
+    if (p.max_split < 1 || p.max_split > kMaxSplit) return CFPP_ERR_DIMS;
+    BatchAttn b{};
+    b.batch = a->batch; b.layer_id = a->layer_id;
+    b.indptr = a->paged_kv_indptr; b.indices = a->paged_kv_indices;
+    b.k_ptrs = reinterpret_cast<const unsigned long long*>(a->k_cache_ptrs);
+    b.v_ptrs = reinterpret_cast<const unsigned long long*>(a->v_cache_ptrs);
+    b.positions = reinterpret_cast<const long long*>(a->positions);
+    b.cos_sin = a->cos_sin;
+    const long long items = (long long)a->batch * d.heads * p.max_split;
+    const int agrid = (int)((items + kStreamers - 1) / kStreamers);
+    hipLaunchKernelGGL(k_batch_attn, dim3(agrid), dim3(kStreamers * 64), 0, st, p, b);
+    if ((rc = (int)hipGetLastError())) return rc;
+
+    BatchGemv o{};
+    o.W = h(a->w_o); o.R = d.hidden; o.K = d.hidden;
+    o.x = reinterpret_cast<const half_t*>(ws + L.attn_vec);
+    o.out_f16 = reinterpret_cast<half_t*>(a->output);
+    o.batch = a->batch;
+    return launch_batch_gemv(nch, o, grid, st);
 }
 
 int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void* attn_output,

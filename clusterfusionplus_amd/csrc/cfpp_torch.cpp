@@ -446,6 +446,76 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> llama_decoder_layer_sglang(Tensor inp
     return std::make_tuple(std::get<0>(r), residual, std::get<1>(r), std::get<2>(r));
 }
 
+// llama_decoder_layer_batch_decode_sglang of the reference (include/pybind.cpp:90-106,282;
+// include/5090/llama/llama_kernel_batch_sglang_dispatch.cu:6-110): same positional arguments, results written into the
+// caller's `output` and `residual_output`, the new K/V rows into the paged caches; returns None.  The reference reads
+// head count and head size from compile-time constants; here they follow from `cos_sin` (its last dimension is the
+// head size).
+void llama_decoder_layer_batch_decode_sglang(Tensor output, Tensor residual_output, Tensor input, Tensor residual,
+                                             Tensor weight_qkv, Tensor weight_o, Tensor paged_kv_indptr, Tensor paged_kv_indices,
+                                             Tensor k_cache_ptrs, Tensor v_cache_ptrs, int64_t layer_id, Tensor rms_input_weight,
+                                             double eps, Tensor positions, Tensor cos_sin) {
+    const char* op = "llama_decoder_layer_batch_decode_sglang";
+    TORCH_CHECK(input.defined() && input.dim() == 2, "input must have shape [batch, hidden]");
+    const int64_t B = input.size(0), H = input.size(1);
+    TORCH_CHECK(B >= 1, "empty batch");
+    check_half(input, "input", B * H, input);
+    check_half(residual, "residual", B * H, input);
+    check_half(output, "output", B * H, input);
+    check_half(residual_output, "residual_output", B * H, input);
+    check_half(weight_qkv, "weight_qkv", 3 * H * H, input);
+    check_half(weight_o, "weight_o", H * H, input);
+    check_half(rms_input_weight, "rms_input_weight", H, input);
+    TORCH_CHECK(cos_sin.defined() && cos_sin.is_cuda() && cos_sin.device() == input.device() && cos_sin.scalar_type() == torch::kFloat32 &&
+                    cos_sin.is_contiguous() && cos_sin.dim() == 2,
+                "cos_sin must be a contiguous float32 tensor [positions, head_dim] on the device of input");
+    const int64_t D = cos_sin.size(1);
+    TORCH_CHECK(D > 0 && H % D == 0, "hidden size ", H, " is not a multiple of the head size ", D, " (cos_sin.size(1))");
+    auto check_index = [&](const Tensor& t, const char* name, torch::ScalarType ty, int64_t min_numel) {
+        TORCH_CHECK(t.defined() && t.is_cuda() && t.device() == input.device() && t.is_contiguous() && t.scalar_type() == ty &&
+                        t.numel() >= min_numel,
+                    name, " must be a contiguous ", c10::toString(ty), " tensor with at least ", min_numel,
+                    " elements on the device of input");
+    };
+    check_index(paged_kv_indptr, "paged_kv_indptr", torch::kInt32, B + 1);
+    check_index(paged_kv_indices, "paged_kv_indices", torch::kInt32, B);
+    TORCH_CHECK(layer_id >= 0, "layer_id is negative");
+    check_index(k_cache_ptrs, "k_cache_ptrs", k_cache_ptrs.defined() ? k_cache_ptrs.scalar_type() : torch::kUInt64, layer_id + 1);
+    check_index(v_cache_ptrs, "v_cache_ptrs", v_cache_ptrs.defined() ? v_cache_ptrs.scalar_type() : torch::kUInt64, layer_id + 1);
+    TORCH_CHECK(k_cache_ptrs.element_size() == 8 && v_cache_ptrs.element_size() == 8, "cache pointer tables must hold 64-bit values");
+    check_index(positions, "positions", torch::kInt64, B);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+    cfpp_llama_batch a{};
+    a.hidden = (int32_t)H; a.heads = (int32_t)(H / D); a.head_dim = (int32_t)D; a.eps = (float)eps;
+    a.batch = (int32_t)B; a.layer_id = (int32_t)layer_id;
+    a.rms_w = rms_input_weight.data_ptr(); a.w_qkv = weight_qkv.data_ptr(); a.w_o = weight_o.data_ptr();
+    a.input = input.data_ptr(); a.residual = residual.data_ptr();
+    a.residual_out = residual_output.data_ptr(); a.output = output.data_ptr();
+    a.paged_kv_indptr = paged_kv_indptr.data_ptr<int32_t>(); a.paged_kv_indices = paged_kv_indices.data_ptr<int32_t>();
+    a.k_cache_ptrs = reinterpret_cast<const uint64_t*>(k_cache_ptrs.data_ptr());
+    a.v_cache_ptrs = reinterpret_cast<const uint64_t*>(v_cache_ptrs.data_ptr());
+    a.positions = positions.data_ptr<int64_t>(); a.cos_sin = cos_sin.data_ptr<float>();
+    const size_t bytes = cfpp_llama_batch_workspace_bytes(a.hidden, a.heads, a.head_dim, a.batch);
+    TORCH_CHECK(bytes > 0, "unsupported layer dimensions (hidden ", H, ", head size ", D, ")");
+    hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    // zero-initialised scratch per (device, stream, geometry, batch): its counters return to zero after every call
+    static std::mutex mu;
+    static std::map<std::tuple<int, void*, int, int, int>, Tensor> cache;
+    Tensor ws;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto key = std::make_tuple((int)input.device().index(), (void*)st, (int)H, (int)D, (int)B);
+        auto it = cache.find(key);
+        if (it == cache.end()) {
+            ws = torch::zeros({(int64_t)bytes + 256}, torch::TensorOptions().dtype(torch::kUInt8).device(input.device()));
+            cache[key] = ws;
+        } else {
+            ws = it->second;
+        }
+    }
+    check_rc(cfpp_llama_batch_decode(&a, ws_ptr(ws), bytes, st), op);
+}
+
 // output = input + W_down (silu(Wg n) * (Wu n)), n = RMSNorm(input) * rms_weight; gate_up_weight = [Wg; Wu] ([2F, H])
 Tensor llama_mlp(Tensor input, Tensor rms_weight, Tensor gate_up_weight, Tensor down_weight, double eps) {
     TORCH_CHECK(input.defined() && input.dim() >= 1, "input is undefined");
@@ -500,6 +570,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("llama_decoder_layer_sglang", &llama_decoder_layer_sglang, py::arg("input"), py::arg("residual"), py::arg("weight_qkv"),
           py::arg("weight_o"), py::arg("k_cache"), py::arg("v_cache"), py::arg("rms_input_weight"), py::arg("eps"), py::arg("cos"),
           py::arg("sin"), py::arg("num_heads") = 32);
+    m.def("llama_decoder_layer_batch_decode_sglang", &llama_decoder_layer_batch_decode_sglang, py::arg("output"),
+          py::arg("residual_output"), py::arg("input"), py::arg("residual"), py::arg("weight_qkv"), py::arg("weight_o"),
+          py::arg("paged_kv_indptr"), py::arg("paged_kv_indices"), py::arg("k_cache_ptrs"), py::arg("v_cache_ptrs"),
+          py::arg("layer_id"), py::arg("rms_input_weight"), py::arg("eps"), py::arg("positions"), py::arg("cos_sin"));
     m.def("llama_mlp", &llama_mlp, py::arg("input"), py::arg("rms_weight"), py::arg("gate_up_weight"), py::arg("down_weight"),
           py::arg("eps"));
     m.def("llama_decoder_layer_full", &llama_decoder_layer_full, py::arg("input"), py::arg("weight_qkv"), py::arg("weight_o"),

@@ -35,7 +35,8 @@ typedef enum cfpp_status {
     CFPP_ERR_CONTEXT = -5,     /* unknown / duplicate context id */
     CFPP_ERR_MODE = -6,        /* unknown mode */
     CFPP_ERR_DEVICE = -7,      /* device-side failure flag raised (bounded wait expired, bad seq_len) */
-    CFPP_ERR_ALIGN = -8        /* a tensor pointer is not 16-byte aligned */
+    CFPP_ERR_ALIGN = -8,       /* a tensor pointer is not 16-byte aligned */
+    CFPP_ERR_ALIAS = -9        /* an output overlaps an input it must not overlap */
 } cfpp_status;
 
 /* Layer geometry.  Pythia-2.8B = {2560,32,80,20,10240,1e-5}, Pythia-6.9B = {4096,32,128,32,16384,1e-5}
@@ -155,6 +156,40 @@ typedef struct cfpp_llama_mlp_args {
 
 size_t cfpp_llama_mlp_workspace_bytes(int32_t hidden, int32_t ffn);
 int cfpp_llama_mlp(const cfpp_llama_mlp_args* m, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- LLaMA attention block for a batch of sequences over paged caches ------------------------------------
+ * Replaces llama_decoder_layer_batch_sglang_sm120 (reference include/pybind.cpp:90-106;
+ * include/5090/llama/llama_kernel_batch_sglang_dispatch.cu:6-110; kernel_batch_sglang.cuh:43-60 arguments, :120-123
+ * page table, :343-367 RoPE from cos_sin[position] and the write of the new K/V row).  For every sequence b:
+ *   r = fp16(input[b] + residual[b]) -> residual_out[b];  n = RMSNorm(r) * rms_w;  [q;k;v] = W_qkv n;  NeoX RoPE over
+ *   the whole head with cos_sin[positions[b]] (D/2 cosines, then D/2 sines);  the new k, v rows are stored in cache
+ *   row paged_kv_indices[paged_kv_indptr[b+1] - 1];  attention over the rows paged_kv_indices[paged_kv_indptr[b] ..
+ *   paged_kv_indptr[b+1] - 1) and the new token;  output[b] = W_o attn (no residual).
+ * Caches are [rows, H] fp16 with head-major columns (page size 1); k_cache_ptrs / v_cache_ptrs are device arrays of
+ * their base addresses per layer, read on the device.  All index arrays live in device memory and are not read by
+ * the host.  residual_out must not alias input or residual (CFPP_ERR_ALIAS).
+ * Workspace: cfpp_llama_batch_workspace_bytes, 256-byte aligned, zero-initialised once, one per stream. */
+typedef struct cfpp_llama_batch {
+    int32_t hidden, heads, head_dim;
+    float eps;
+    int32_t batch, layer_id;
+    const void* rms_w;                /* [H] fp16 */
+    const void* w_qkv;                /* [3H, H] fp16 = [Wq; Wk; Wv] */
+    const void* w_o;                  /* [H, H] fp16 */
+    const void* input;                /* [batch, H] fp16 */
+    const void* residual;             /* [batch, H] fp16 */
+    void* residual_out;               /* [batch, H] fp16 */
+    void* output;                     /* [batch, H] fp16 */
+    const int32_t* paged_kv_indptr;   /* [batch + 1] */
+    const int32_t* paged_kv_indices;  /* [paged_kv_indptr[batch]] cache rows */
+    const uint64_t* k_cache_ptrs;     /* [layers] */
+    const uint64_t* v_cache_ptrs;     /* [layers] */
+    const int64_t* positions;         /* [batch] */
+    const float* cos_sin;             /* [max_position, D] fp32 */
+} cfpp_llama_batch;
+
+size_t cfpp_llama_batch_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim, int32_t batch);
+int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Second half: output = input + attn_output + W_down mlp_intermediate + b_down.
  * Replaces pythia_2b8_mlp_only_sm120 (reference include/pybind.cpp:174-180;

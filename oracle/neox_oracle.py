@@ -311,6 +311,41 @@ def llama_attention_sglang(
     return {"output": out, "residual": r, "k_new": k_new[None], "v_new": v_new[None], "attn_heads": o}
 
 
+def llama_batch_decode_paged(
+    x: torch.Tensor,
+    residual: torch.Tensor,
+    w: Dict[str, torch.Tensor],
+    indptr: torch.Tensor,
+    indices: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    positions: torch.Tensor,
+    cos_sin: torch.Tensor,
+    dims: LlamaDims,
+    dtype: torch.dtype = torch.float32,
+    round_io: bool = True,
+) -> Dict[str, torch.Tensor]:
+    """One decode step of a batch of sequences over paged caches (`llama_decoder_layer_batch_decode_sglang`,
+    reference include/5090/llama/kernel_batch_sglang.cuh): sequence b owns the cache rows
+    indices[indptr[b] : indptr[b+1]]; the last of them receives the new token's K/V (:367-370, end_idx =
+    indptr[b+1]-1 at :120-122), the others are attended over together with the new token; RoPE angles come from
+    cos_sin[positions[b]] = [cos(D/2) | sin(D/2)] (:343-346).  Per sequence this is `llama_attention_sglang` on the
+    gathered rows.  `x`, `residual` [B,H]; caches [rows,H] (copies are updated and returned)."""
+    B, H, D = x.shape[0], dims.hidden, dims.head_dim
+    k_cache, v_cache = k_cache.clone(), v_cache.clone()
+    outs, ress = [], []
+    for b in range(B):
+        lo, hi = int(indptr[b]), int(indptr[b + 1]) - 1
+        rows = indices[lo:hi].long()
+        cs = cos_sin[int(positions[b])].float()
+        r = llama_attention_sglang(x[b:b + 1], residual[b:b + 1], w, k_cache[rows], v_cache[rows], cs[: D // 2], cs[D // 2:], dims, dtype, round_io)
+        outs.append(r["output"]); ress.append(r["residual"])
+        slot = int(indices[hi])
+        k_cache[slot] = r["k_new"].reshape(H).to(k_cache.dtype)
+        v_cache[slot] = r["v_new"].reshape(H).to(v_cache.dtype)
+    return {"output": torch.cat(outs), "residual": torch.cat(ress), "k_cache": k_cache, "v_cache": v_cache}
+
+
 def make_llama_attn_inputs(dims: LlamaDims, S: int, seed: int = 0, w_std: float = 0.02):
     """Seeded fp16 tensors for the LLaMA attention block: weights dict, input, residual, caches [S,H], cos/sin [1,D]
     (random angles per pair, duplicated halves, as reference tests/test_llama.py:24-28,140-142 builds them)."""

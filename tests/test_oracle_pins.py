@@ -269,3 +269,50 @@ def test_llama_attention_closed_forms():
     got3 = O.llama_attention_sglang(x, None, w, k, v, one, zero, dims, dtype=torch.float64, round_io=False)
     n = O.rms_norm(x.double(), w["rms1"].double(), dims.eps)
     assert torch.allclose(got3["k_new"].reshape(-1), (n @ w["w_qkv"].double().t()).reshape(3, -1)[1], atol=1e-12, rtol=0)
+
+
+def test_llama_batch_decode_paged_matches_hf_per_sequence():
+    """Page-table conventions of the batched op, against HF modules fed by hand: the sequence's history is the rows
+    indices[indptr[b] : indptr[b+1]-1], the new K/V lands in row indices[indptr[b+1]-1], and the angles of position p
+    are row p of cos_sin = [cos | sin] — here HF's own LlamaRotaryEmbedding evaluated at that position."""
+    hf = pytest.importorskip("transformers")
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding
+    from oracle import hf_neox
+    dims, _, w, _, _, _, _, _, _ = _tiny_llama()
+    H, D = dims.hidden, dims.head_dim
+    g = torch.Generator().manual_seed(5)
+    lens = [5, 0, 9]
+    B, pool, max_pos = len(lens), 40, 64
+    x = torch.randn(B, H, generator=g).half()
+    res = torch.randn(B, H, generator=g).half()
+    k = torch.randn(pool, H, generator=g).half()
+    v = torch.randn(pool, H, generator=g).half()
+    indices = torch.randperm(pool, generator=g)[: sum(lens) + B].to(torch.int32)
+    indptr = torch.tensor([0, 6, 7, 17], dtype=torch.int32)
+    positions = torch.tensor([5, 63, 20], dtype=torch.int64)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2).double() / D))
+    ang = torch.arange(max_pos).double()[:, None] * inv[None, :]
+    cos_sin = torch.cat([torch.cos(ang), torch.sin(ang)], dim=-1)
+    got = O.llama_batch_decode_paged(x, res, w, indptr, indices, k, v, positions, cos_sin, dims, dtype=torch.float64, round_io=False)
+
+    layer = hf_neox.build_hf_llama_layer(dims, w, dtype=torch.float64)
+    cfg = LlamaConfig(hidden_size=H, num_attention_heads=dims.heads, head_dim=D, max_position_embeddings=max_pos, rope_theta=10000.0)
+    rotary = LlamaRotaryEmbedding(cfg)
+    touched = []
+    for b in range(B):
+        lo, hi = int(indptr[b]), int(indptr[b + 1]) - 1
+        rows = indices[lo:hi].long()
+        hc, hs = rotary(torch.zeros(1, 1, H, dtype=torch.float64), positions[b].reshape(1, 1))     # [1,1,D] each
+        r = (x[b:b + 1].double() + res[b:b + 1].double()).half().double()
+        want, k_new, v_new = hf_neox.hf_llama_attention(layer, r, k[rows], v[rows], hc, hs, dims, dtype=torch.float64)
+        assert torch.allclose(got["output"][b:b + 1].double(), want, atol=1e-6, rtol=0)      # HF takes norm and softmax in float32
+        slot = int(indices[hi])
+        touched.append(slot)
+        # the caches hold fp16
+        assert torch.equal(got["k_cache"][slot], k_new.reshape(-1).half()) or torch.allclose(got["k_cache"][slot].double(), k_new.reshape(-1), atol=0, rtol=1e-3)
+        assert torch.allclose(got["v_cache"][slot].double(), v_new.reshape(-1), atol=1e-6, rtol=1e-3)
+        assert torch.equal(got["residual"][b:b + 1].double(), r)
+    keep = torch.ones(pool, dtype=torch.bool)
+    keep[touched] = False
+    assert torch.equal(got["k_cache"][keep], k[keep]) and torch.equal(got["v_cache"][keep], v[keep])
