@@ -858,15 +858,31 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
         }
         m = mt;
     };
-    if (it.ntiles > 0) process(it.t0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    if (it.ntiles > 2) attn_load_tile<PAGED>(p, it, it.t0, 2, lane);     // the third tile travels while the second is reduced
-    __builtin_amdgcn_sched_barrier(0);
-    if (it.ntiles > 1) process(it.t1, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    for (int i = 2; i < it.ntiles; ++i) {
-        if (i != 2) attn_load_tile<PAGED>(p, it, it.t0, i, lane);
-        process(it.t0, i);
+    if (PAGED) {
+        // items of a batched launch can be long: keep two tiles in flight all the way
+        for (int i = 0; i < it.ntiles; i += 2) {
+            process(it.t0, i);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + 2 < it.ntiles) attn_load_tile<PAGED>(p, it, it.t0, i + 2, lane);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + 1 < it.ntiles) {
+                process(it.t1, i + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                if (i + 3 < it.ntiles) attn_load_tile<PAGED>(p, it, it.t1, i + 3, lane);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    } else {
+        if (it.ntiles > 0) process(it.t0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (it.ntiles > 2) attn_load_tile<PAGED>(p, it, it.t0, 2, lane);     // the third tile travels while the second is reduced
+        __builtin_amdgcn_sched_barrier(0);
+        if (it.ntiles > 1) process(it.t1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        for (int i = 2; i < it.ntiles; ++i) {
+            if (i != 2) attn_load_tile<PAGED>(p, it, it.t0, i, lane);
+            process(it.t0, i);
+        }
     }
 
     // merge the four groups (lanes sub, sub+16, sub+32, sub+48 hold the same dims)

@@ -581,21 +581,55 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_gemv(BatchGemv a) {
         }
         __syncthreads();
         int prow = 0;
-        auto consume = [&](const RowTile<NCH, RPI>& t, int valid) {
-            for (int tk = 0; tk < nb; ++tk) {
-                half2_t xv[NCH][4];
+        // Sequences are taken two at a time and every dot product is split over two accumulators, so that eight
+        // independent chains of dot instructions (and four independent reductions) are in flight: with one wave
+        // per SIMD nothing else hides their latencies.
+        auto fetch_x = [&](int tk, half2_t (&xv)[NCH][4]) {
 #pragma unroll
-                for (int i = 0; i < NCH; ++i) {
-                    const u32x4 q = *reinterpret_cast<const u32x4*>(&xs[tk][i * kChunk + lane * 8]);
-                    xv[i][0] = as_h2(q.x); xv[i][1] = as_h2(q.y); xv[i][2] = as_h2(q.z); xv[i][3] = as_h2(q.w);
+            for (int i = 0; i < NCH; ++i) {
+                const u32x4 q = *reinterpret_cast<const u32x4*>(&xs[tk][i * kChunk + lane * 8]);
+                xv[i][0] = as_h2(q.x); xv[i][1] = as_h2(q.y); xv[i][2] = as_h2(q.z); xv[i][3] = as_h2(q.w);
+            }
+        };
+        auto consume = [&](const RowTile<NCH, RPI>& t, int valid) {
+            int tk = 0;
+            for (; tk + 2 <= nb; tk += 2) {
+                half2_t xa[NCH][4], xb[NCH][4];
+                fetch_x(tk, xa);
+                fetch_x(tk + 1, xb);
+                float acc[RPI][2][2];
+#pragma unroll
+                for (int j = 0; j < RPI; ++j) {
+                    acc[j][0][0] = acc[j][0][1] = acc[j][1][0] = acc[j][1][1] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < NCH; ++i) {
+                        acc[j][0][i & 1] = dot8(t.w[j][i], xa[i], acc[j][0][i & 1]);
+                        acc[j][1][i & 1] = dot8(t.w[j][i], xb[i], acc[j][1][i & 1]);
+                    }
                 }
 #pragma unroll
                 for (int j = 0; j < RPI; ++j) {
-                    float acc = 0.f;
+                    const float ra = wave_sum(acc[j][0][0] + acc[j][0][1]);
+                    const float rb = wave_sum(acc[j][1][0] + acc[j][1][1]);
+                    if (j < valid && lane == 0) {
+                        park[wave][tk * kBatchParkRows + prow + j] = ra;
+                        park[wave][(tk + 1) * kBatchParkRows + prow + j] = rb;
+                    }
+                }
+            }
+            if (tk < nb) {
+                half2_t xa[NCH][4];
+                fetch_x(tk, xa);
 #pragma unroll
-                    for (int i = 0; i < NCH; ++i) acc = dot8(t.w[j][i], xv[i], acc);
-                    acc = wave_sum(acc);
-                    if (j < valid && lane == 0) park[wave][tk * kBatchParkRows + prow + j] = acc;
+                for (int j = 0; j < RPI; ++j) {
+                    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+                    for (int i = 0; i < NCH; ++i) {
+                        if (i & 1) a1 = dot8(t.w[j][i], xa[i], a1);
+                        else a0 = dot8(t.w[j][i], xa[i], a0);
+                    }
+                    const float ra = wave_sum(a0 + a1);
+                    if (j < valid && lane == 0) park[wave][tk * kBatchParkRows + prow + j] = ra;
                 }
             }
             prow += valid;
@@ -627,6 +661,110 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_gemv(BatchGemv a) {
             const size_t o = (size_t)(t0 + tk) * a.R + rw.first + r;
             if (a.out_f32 != nullptr) a.out_f32[o] = val;
             else a.out_f16[o] = (half_t)val;
+        }
+    }
+}
+
+// The same products on the matrix cores: from about eight sequences on, the dot-instruction kernel above is bound
+// by its arithmetic, not by the weight stream.  A workgroup owns 16 weight rows; its eight waves split the row
+// length, and each wave requests its whole share (16 rows x K/8) at once.  v_mfma_f32_16x16x32_f16 then multiplies
+// that 16 x 32 weight block with the matching 32 x 16 block of the (normalised) input rows of 16 sequences; lane l
+// supplies row l % 16 and the eight k values of group l / 16 for both operands, so both are loaded with the same
+// address pattern.  The input rows come from global memory (every workgroup reads the same few rows: cache hits).
+// The weights stay in registers while further groups of 16 sequences are processed.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+struct BatchMfma {
+    const half_t* W; int R, K;         // weight rows [R, K]; R % 16 == 0, K % 256 == 0
+    const half_t* x;                   // [batch][K]
+    float* out_f32; half_t* out_f16;   // [batch][R], one of the two
+    int batch;
+};
+template <int KSTEPS>
+__global__ __launch_bounds__(512) void k_batch_mfma(BatchMfma a) {
+    __shared__ f32x4_t red[8][64];
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int r0 = blockIdx.x * 16;
+    const size_t koff = (size_t)wave * (a.K / 8) + 8 * (lane >> 4);
+    const half_t* wp = a.W + (size_t)(r0 + (lane & 15)) * a.K + koff;
+    u32x4 w[KSTEPS];
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) w[s] = ld_stream16(wp + 32 * s);
+    for (int t0 = 0; t0 < a.batch; t0 += 16) {
+        const int tok = t0 + (lane & 15) < a.batch ? t0 + (lane & 15) : a.batch - 1;
+        const half_t* xp = a.x + (size_t)tok * a.K + koff;
+        u32x4 x[KSTEPS];
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) x[s] = ld16(xp + 32 * s);
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, w[s]), __builtin_bit_cast(half8_t, x[s]), acc, 0, 0, 0);
+        __syncthreads();      // the previous group's partial sums have been read
+        red[wave][lane] = acc;
+        __syncthreads();
+        // acc[i] of lane l belongs to weight row r0 + 4 (l / 16) + i and sequence t0 + l % 16; wave i adds up element i
+        if (wave < 4) {
+            float sum = 0.f;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sum += red[u][lane][wave];
+            const int seq = t0 + (lane & 15), row = r0 + 4 * (lane >> 4) + wave;
+            if (seq < a.batch) {
+                const size_t o = (size_t)seq * a.R + row;
+                if (a.out_f32 != nullptr) a.out_f32[o] = sum;
+                else a.out_f16[o] = (half_t)sum;
+            }
+        }
+    }
+}
+
+// Fused add + RMSNorm of the input rows, one wave per sequence: y = fp16(r * rstd * w), r = fp16(x + x_add) -> sum_out.
+struct BatchNorm {
+    const half_t *x, *x_add, *norm_w;
+    half_t *sum_out, *y;
+    float eps;
+    int K, batch;
+};
+template <int NCH>
+__global__ __launch_bounds__(kStreamers * 64) void k_batch_norm(BatchNorm a) {
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int seq = blockIdx.x * kStreamers + wave;
+    if (seq >= a.batch) return;
+    const size_t base = (size_t)seq * a.K;
+    float v[NCH][8];
+    float ss = 0.f;
+    u32x4 gw[NCH];       // the norm weights travel together with the rows
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int col = i * kChunk + lane * 8;
+        gw[i] = ld16(a.norm_w + (col < a.K ? col : 0));
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int col = i * kChunk + lane * 8;
+        const bool in = col < a.K;
+        u32x4 r = {0u, 0u, 0u, 0u}, ra = {0u, 0u, 0u, 0u};
+        if (in) { r = ld16(a.x + base + col); ra = ld16(a.x_add + base + col); }
+        float w[8];
+        unpack8(r, v[i]); unpack8(ra, w);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] += w[j];
+        r = pack8(v[i]);
+        unpack8(r, v[i]);
+        if (in) *reinterpret_cast<u32x4*>(a.sum_out + base + col) = r;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += v[i][j] * v[i][j];
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)a.K + a.eps);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int col = i * kChunk + lane * 8;
+        if (col < a.K) {
+            float g[8];
+            unpack8(gw[i], g);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[i][j] = v[i][j] * rstd * g[j];
+            *reinterpret_cast<u32x4*>(a.y + base + col) = pack8(v[i]);
         }
     }
 }
@@ -957,13 +1095,14 @@ int run_split(const Plan& pl, LayerParams& p, int seq_hint, hipStream_t st) {
 // =================================================================================================
 // ---- launchers of the batched LLaMA attention block ---------------------------------------------------
 namespace {
-struct BatchLayout { size_t qkv_raw, attn_vec, k_new, v_new, part_ml, part_acc, head_cnt, bar, total; };
+struct BatchLayout { size_t qkv_raw, x_norm, attn_vec, k_new, v_new, part_ml, part_acc, head_cnt, bar, total; };
 BatchLayout batch_layout(const cfpp_neox_dims& d, int batch) {
     BatchLayout w{};
     size_t off = 0;
     auto take = [&](size_t bytes) { const size_t at = off; off += align_up(bytes, 256); return at; };
     const size_t B = (size_t)batch, H = (size_t)d.hidden;
     w.qkv_raw = take(B * 3 * H * 4);
+    w.x_norm = take(B * H * 2);
     w.attn_vec = take(B * H * 2);
     w.k_new = take(B * H * 2);
     w.v_new = take(B * H * 2);
@@ -978,6 +1117,29 @@ template <int NCH>
 int launch_batch_gemv_t(const BatchGemv& a, int grid, hipStream_t st) {
     if (a.K == NCH * kChunk) hipLaunchKernelGGL((k_batch_gemv<NCH, true>), dim3(grid), dim3(kStreamers * 64), 0, st, a);
     else hipLaunchKernelGGL((k_batch_gemv<NCH, false>), dim3(grid), dim3(kStreamers * 64), 0, st, a);
+    return (int)hipGetLastError();
+}
+int launch_batch_mfma(const BatchMfma& a, hipStream_t st) {
+    const int grid = a.R / 16;
+    switch (a.K / 256) {
+        case 4: hipLaunchKernelGGL((k_batch_mfma<4>), dim3(grid), dim3(512), 0, st, a); break;
+        case 8: hipLaunchKernelGGL((k_batch_mfma<8>), dim3(grid), dim3(512), 0, st, a); break;
+        case 16: hipLaunchKernelGGL((k_batch_mfma<16>), dim3(grid), dim3(512), 0, st, a); break;
+        default: return CFPP_ERR_DIMS;
+    }
+    return (int)hipGetLastError();
+}
+bool batch_mfma_supported(int rows, int k) { return rows % 16 == 0 && k % 256 == 0 && (k == 1024 || k == 2048 || k == 4096); }
+int launch_batch_norm(int nch, const BatchNorm& a, hipStream_t st) {
+    const dim3 grid((a.batch + kStreamers - 1) / kStreamers), block(kStreamers * 64);
+    switch (nch) {
+        case 1: hipLaunchKernelGGL((k_batch_norm<1>), grid, block, 0, st, a); break;
+        case 2: hipLaunchKernelGGL((k_batch_norm<2>), grid, block, 0, st, a); break;
+        case 4: hipLaunchKernelGGL((k_batch_norm<4>), grid, block, 0, st, a); break;
+        case 5: hipLaunchKernelGGL((k_batch_norm<5>), grid, block, 0, st, a); break;
+        case 8: hipLaunchKernelGGL((k_batch_norm<8>), grid, block, 0, st, a); break;
+        default: return CFPP_ERR_DIMS;
+    }
     return (int)hipGetLastError();
 }
 int launch_batch_gemv(int nch, const BatchGemv& a, int grid, hipStream_t st) {
@@ -1160,20 +1322,37 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
     const BatchLayout L = batch_layout(d, a->batch);
     if (workspace_bytes < L.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CFPP_ERR_WORKSPACE;
     const int nch = (d.hidden + kChunk - 1) / kChunk;
-    const int grid = streaming_grid();
+    // two workgroups per compute unit for the row streams: a second wave per SIMD covers the latencies of the
+    // per-sequence reductions
+    const int grid = streaming_grid() * env_int("CFPP_BATCH_WGS_PER_CU", 2);
     const int waves = grid * kStreamers;
-    if ((3 * d.hidden + waves - 1) / waves + 2 > kBatchParkRows) return CFPP_ERR_DIMS;
+    if (grid < 1 || (3 * d.hidden + waves - 1) / waves + 2 > kBatchParkRows) return CFPP_ERR_DIMS;
     char* ws = reinterpret_cast<char*>(workspace);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     auto h = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
 
+    // matrix-core kernels where the geometry allows (and from two sequences on: a single sequence is served as
+    // well by the dot-instruction kernel, without the separate norm launch)
+    const bool mfma = batch_mfma_supported(d.hidden, d.hidden) && a->batch >= env_int("CFPP_BATCH_MFMA_FROM", 2);
+    if (mfma) {
+        BatchNorm n{};
+        n.x = h(a->input); n.x_add = h(a->residual); n.norm_w = h(a->rms_w);
+        n.sum_out = reinterpret_cast<half_t*>(a->residual_out); n.y = reinterpret_cast<half_t*>(ws + L.x_norm);
+        n.eps = a->eps; n.K = d.hidden; n.batch = a->batch;
+        if ((rc = launch_batch_norm(nch, n, st))) return rc;
+        BatchMfma m{};
+        m.W = h(a->w_qkv); m.R = 3 * d.hidden; m.K = d.hidden;
+        m.x = reinterpret_cast<const half_t*>(ws + L.x_norm);
+        m.out_f32 = reinterpret_cast<float*>(ws + L.qkv_raw); m.out_f16 = nullptr; m.batch = a->batch;
+        if ((rc = launch_batch_mfma(m, st))) return rc;
+    }
     BatchGemv g{};
     g.W = h(a->w_qkv); g.R = 3 * d.hidden; g.K = d.hidden;
     g.x = h(a->input); g.x_add = h(a->residual); g.sum_out = reinterpret_cast<half_t*>(a->residual_out);
     g.norm_w = h(a->rms_w); g.eps = a->eps;
     g.out_f32 = reinterpret_cast<float*>(ws + L.qkv_raw); g.out_f16 = nullptr;
     g.batch = a->batch;
-    if ((rc = launch_batch_gemv(nch, g, grid, st))) return rc;
+    if (!mfma && (rc = launch_batch_gemv(nch, g, grid, st))) return rc;
 
     LayerParams p{};
     p.H = d.hidden; p.heads = d.heads; p.D = d.head_dim; p.rot = d.head_dim; p.F = 0;
@@ -1190,7 +1369,7 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
     p.qkv_head_stride = d.head_dim; p.qkv_k_off = d.hidden; p.qkv_v_off = 2 * d.hidden;
     p.append_kv = 1;
     // enough (sequence, head, split) items to fill the attention waves about twice, and no more
-    int ms = (2 * waves) / (a->batch * d.heads);
+    int ms = (2 * streaming_grid() * kStreamers) / (a->batch * d.heads);
     ms = ms < 1 ? 1 : (ms > 32 ? 32 : ms);
     p.max_split = env_int("CFPP_MAX_SPLIT", ms);
     if (p.max_split < 1 || p.max_split > kMaxSplit) return CFPP_ERR_DIMS;
@@ -1211,6 +1390,11 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
     o.x = reinterpret_cast<const half_t*>(ws + L.attn_vec);
     o.out_f16 = reinterpret_cast<half_t*>(a->output);
     o.batch = a->batch;
+    if (mfma) {
+        BatchMfma m{};
+        m.W = o.W; m.R = o.R; m.K = o.K; m.x = o.x; m.out_f32 = nullptr; m.out_f16 = o.out_f16; m.batch = o.batch;
+        return launch_batch_mfma(m, st);
+    }
     return launch_batch_gemv(nch, o, grid, st);
 }
 
