@@ -175,12 +175,73 @@ def bench_llama_layer(args):
         "cpu_baseline": None}), flush=True)
 
 
+def bench_llama_batch(args):
+    """Extra workload (not the headline): the LLaMA-2-7B attention block for --batch sequences of --ctx cached tokens
+    each over paged caches (the reference's llama_decoder_layer_batch_decode_sglang), pages scattered over the pool,
+    six weight sets in turn so that every call reads HBM-cold weights."""
+    import torch
+    import clusterfusion as cf
+    from oracle import neox_oracle as O      # geometry constants only
+    dev = "cuda:0"
+    dims, S, B, nset = O.LLAMA2_7B, args.ctx, args.batch, 6
+    H, D = dims.hidden, dims.head_dim
+    g = torch.Generator().manual_seed(2)
+    ws = [((0.02 * torch.randn(3 * H, H, generator=g)).half().to(dev), (0.02 * torch.randn(H, H, generator=g)).half().to(dev))
+          for _ in range(nset)]
+    rms = (1 + 0.1 * torch.randn(H, generator=g)).half().to(dev)
+    max_pos = S + 1
+    inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2).float() / D))
+    ang = torch.arange(max_pos).float()[:, None] * inv[None, :]
+    cos_sin = torch.cat([torch.cos(ang), torch.sin(ang)], dim=-1).float().contiguous().to(dev)
+    total = B * (S + 1)
+    pool = total + 64
+    ncache = 4 if B * S <= 32768 else 2
+    caches = [(torch.randn(pool, H, generator=g).half().to(dev), torch.randn(pool, H, generator=g).half().to(dev)) for _ in range(ncache)]
+    kptr = torch.tensor([a.data_ptr() for a, _ in caches], dtype=torch.uint64, device=dev)
+    vptr = torch.tensor([b.data_ptr() for _, b in caches], dtype=torch.uint64, device=dev)
+    indices = torch.randperm(pool, generator=g)[:total].to(torch.int32).to(dev)
+    indptr = (torch.arange(B + 1) * (S + 1)).to(torch.int32).to(dev)
+    pos = torch.full((B,), S, dtype=torch.int64, device=dev)
+    x = torch.randn(B, H, generator=g).half().to(dev)
+    res = torch.randn(B, H, generator=g).half().to(dev)
+    out, res_out = torch.empty_like(x), torch.empty_like(x)
+
+    def call(i):
+        wq, wo = ws[i % nset]
+        cf.llama_decoder_layer_batch_decode_sglang(out, res_out, x, res, wq, wo, indptr, indices, kptr, vptr, i % ncache, rms, dims.eps,
+                                                   pos, cos_sin)
+    for i in range(max(args.warmup, nset)):
+        call(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(args.steps):
+        call(i)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / args.steps
+    nbytes = 2 * 4 * H * H + 2 * H + B * S * 2 * H * 2
+    gbps = nbytes / (us * 1e-6) / 1e9
+    print(json.dumps({
+        "metric": "batch_step_latency_us", "value": round(us, 2), "unit": "us/call", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us * 1e-3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"llama2_7b attention block, {B} sequences x {S} cached tokens over paged caches (page = 1 token, "
+                               "scattered), 4 launches per call", "batch": B, "context": S, "hidden": H,
+                   "tokens_per_s_per_layer": round(B / (us * 1e-6))},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "traffic": None, "kernel": "k_batch_norm + k_batch_mfma_lds (QKV) + k_batch_attn + k_batch_mfma_lds (O)",
+                     "bytes_per_launch": nbytes, "launch_us": round(us, 2)},
+        "cpu_baseline": None}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8", "llama2_7b_layer"])
+    ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8", "llama2_7b_layer", "llama2_7b_batch"])
+    ap.add_argument("--batch", type=int, default=16, help="sequences per call (llama2_7b_batch only)")
     ap.add_argument("--ctx", type=int, default=2048, help="KV-cache rows already filled when the timed region starts")
     ap.add_argument("--mode", default="fused", choices=["fused", "split"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -200,6 +261,10 @@ def main():
         if args.ctx == 2048:
             args.ctx = 4096          # the context this workload is quoted at
         return bench_llama_layer(args)
+    if args.model == "llama2_7b_batch":
+        if args.ctx == 2048:
+            args.ctx = 1024
+        return bench_llama_batch(args)
     cfg = pkg.PYTHIA_6B9 if args.model == "pythia_6b9" else pkg.PYTHIA_2B8
     K, W = args.steps, args.warmup
     rows = args.ctx + W + K + 40
