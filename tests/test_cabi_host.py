@@ -41,8 +41,8 @@ def test_status_strings_and_version(lib):
     lib.cfpp_status_str.restype = ctypes.c_char_p
     lib.cfpp_version.restype = ctypes.c_char_p
     assert lib.cfpp_status_str(0) == b"ok"
-    seen = {lib.cfpp_status_str(-i) for i in range(1, 9)}
-    assert len(seen) == 8 and b"unknown status" not in seen
+    seen = {lib.cfpp_status_str(-i) for i in range(1, 10)}
+    assert len(seen) == 9 and b"unknown status" not in seen
     assert b"gfx950" in lib.cfpp_version()
 
 
@@ -76,12 +76,45 @@ def test_null_and_mode_errors_launch_nothing(lib):
     assert lib.cfpp_neox_lm_head(4096, 100, ctypes.c_float(1e-5), None, None, None, None, None, None) == -1
 
 
+class LlamaBatch(ctypes.Structure):
+    _fields_ = [("hidden", ctypes.c_int32), ("heads", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("eps", ctypes.c_float),
+                ("batch", ctypes.c_int32), ("layer_id", ctypes.c_int32)] + [(n, ctypes.c_void_p) for n in (
+                    "rms_w", "w_qkv", "w_o", "input", "residual", "residual_out", "output", "paged_kv_indptr", "paged_kv_indices",
+                    "k_cache_ptrs", "v_cache_ptrs", "positions", "cos_sin")]
+
+
+def test_llama_batch_argument_checks_launch_nothing(lib):
+    lib.cfpp_llama_batch_workspace_bytes.restype = ctypes.c_size_t
+    n = lib.cfpp_llama_batch_workspace_bytes(4096, 32, 128, 16)
+    assert n > 0 and n % 256 == 0
+    assert lib.cfpp_llama_batch_workspace_bytes(4096, 32, 128, 32) > n           # scratch grows with the batch
+    assert lib.cfpp_llama_batch_workspace_bytes(4096, 32, 128, 0) == 0
+    assert lib.cfpp_llama_batch_workspace_bytes(4100, 32, 128, 4) == 0
+    ws = ctypes.c_void_p(256)
+    a = LlamaBatch(4096, 32, 128, 1e-6, 4, 0)
+    assert lib.cfpp_llama_batch_decode(None, ws, ctypes.c_size_t(n), None) == -1
+    assert lib.cfpp_llama_batch_decode(ctypes.byref(a), ws, ctypes.c_size_t(n), None) == -1          # NULL tensors
+    for f in ("rms_w", "w_qkv", "w_o", "input", "residual", "residual_out", "output", "cos_sin", "paged_kv_indptr", "paged_kv_indices",
+              "k_cache_ptrs", "v_cache_ptrs", "positions"):
+        setattr(a, f, 4096)
+    a.residual_out = 8192
+    a.input = 4104                                                                                     # not 16-byte aligned
+    assert lib.cfpp_llama_batch_decode(ctypes.byref(a), ws, ctypes.c_size_t(n), None) == -8
+    a.input = 8192                                                                                     # sum written over a row still read
+    assert lib.cfpp_llama_batch_decode(ctypes.byref(a), ws, ctypes.c_size_t(n), None) == -9
+    a.input = 4096
+    assert lib.cfpp_llama_batch_decode(ctypes.byref(a), ws, ctypes.c_size_t(16), None) == -4           # workspace too small
+    a.batch = 0
+    assert lib.cfpp_llama_batch_decode(ctypes.byref(a), ws, ctypes.c_size_t(n), None) == -2
+
+
 def test_package_imports_and_exposes_reference_names():
     import clusterfusion
     want = ["pythia_2b8_decoder_layer", "pythia_2b8_decoder_layer_split", "pythia_2b8_attention_only",
             "pythia_2b8_mlp_only", "pythia_2b8_create_graph_context", "pythia_2b8_graph_decode_step",
             "pythia_2b8_destroy_graph_context", "pythia_6b9_decoder_layer", "pythia_6b9_create_graph_context",
-            "pythia_6b9_graph_decode_step", "pythia_6b9_destroy_graph_context"]   # reference include/pybind.cpp:284-297
+            "pythia_6b9_graph_decode_step", "pythia_6b9_destroy_graph_context",   # reference include/pybind.cpp:284-297
+            "llama_decoder_layer_sglang", "llama_decoder_layer_batch_decode_sglang"]  # :281-282
     for n in want:
         assert callable(getattr(clusterfusion, n)), n
     # CPU tensors are refused with an exception, not a crash
