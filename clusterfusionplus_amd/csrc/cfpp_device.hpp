@@ -688,7 +688,10 @@ struct StageARpi { static constexpr int value = (16 / NCH) > 0 ? (16 / NCH) : 1;
 // A lane produces dims d0 .. d0+7.  rope_coeffs fetches cos and the signed sin of those dims (1 and 0 for
 // dims >= rot): they do not depend on the layer's own results, so they can be requested early.
 // rope_load8 requests the lane's own values and their rotation partners together (one memory round trip).
+// PAIRS: dim d rotates with d +- rot/2 (false, NeoX) or with its neighbour d ^ 1 (true, GPT-J: even dims take
+// -sin, odd dims +sin, and the tables are indexed by the dim itself; reference include/5090/llama/kernel.cuh:280-313).
 struct RopeCoeffs { float c[8], sg[8]; };
+template <bool PAIRS = false>
 __device__ __forceinline__ void rope_coeffs(int d0, int rot, const float* __restrict__ cs, const float* __restrict__ sn,
                                             bool act, RopeCoeffs& rc) {
     const int hr = rot >> 1;
@@ -696,11 +699,17 @@ __device__ __forceinline__ void rope_coeffs(int d0, int rot, const float* __rest
     for (int j = 0; j < 8; ++j) {
         const int d = d0 + j;
         const bool rotd = act && d < rot;
-        const int t = d < hr ? d : d - hr;       // both halves use the angle of the pair (entries [0, rot/2) of the table)
-        rc.c[j] = rotd ? cs[t] : 1.f;
-        rc.sg[j] = rotd ? (d < hr ? -sn[t] : sn[t]) : 0.f;
+        if (PAIRS) {
+            rc.c[j] = rotd ? cs[d] : 1.f;
+            rc.sg[j] = rotd ? ((d & 1) ? sn[d] : -sn[d]) : 0.f;
+        } else {
+            const int t = d < hr ? d : d - hr;       // both halves use the angle of the pair (entries [0, rot/2) of the table)
+            rc.c[j] = rotd ? cs[t] : 1.f;
+            rc.sg[j] = rotd ? (d < hr ? -sn[t] : sn[t]) : 0.f;
+        }
     }
 }
+template <bool PAIRS = false>
 __device__ __forceinline__ void rope_load8(const float* __restrict__ v, int d0, int rot, const RopeCoeffs& rc, bool act,
                                            float (&out)[8]) {
     float a[8], pr[8];
@@ -710,9 +719,13 @@ __device__ __forceinline__ void rope_load8(const float* __restrict__ v, int d0, 
         ld_agent2(v + d0 + 4, a[4], a[5]); ld_agent2(v + d0 + 6, a[6], a[7]);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const int d = d0 + j;
-            const int pd = d < rot ? (d < hr ? d + hr : d - hr) : d;
-            pr[j] = ld_agent(v + pd);
+            if (PAIRS) {
+                pr[j] = a[j ^ 1];                    // the neighbour is one of the lane's own eight dims
+            } else {
+                const int d = d0 + j;
+                const int pd = d < rot ? (d < hr ? d + hr : d - hr) : d;
+                pr[j] = ld_agent(v + pd);
+            }
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) out[j] = d0 + j < rot ? a[j] * rc.c[j] + pr[j] * rc.sg[j] : a[j];
@@ -762,7 +775,7 @@ __device__ __forceinline__ void attn_load_tile(const LayerParams& p, const AttnI
         kv.v[t] = ld16(vc + (size_t)row * p.H);
     }
 }
-template <bool PAGED = false>
+template <bool PAGED = false, bool PAIRS = false>
 __device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it, int head, int sp, int nsplit, int S, int lane) {
     it.head = head; it.sp = sp; it.nsplit = nsplit; it.S = S;
     const int chunk = (S + nsplit - 1) / nsplit;
@@ -775,11 +788,11 @@ __device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it
     const bool act = sub * 8 < p.D;
     const float* __restrict__ cs = p.cos + (size_t)S * p.rope_stride;   // stride 0: the row is the position
     const float* __restrict__ sn = p.sin + (size_t)S * p.rope_stride;
-    rope_coeffs(act ? sub * 8 : 0, p.rot, cs, sn, act, it.rc);
+    rope_coeffs<PAIRS>(act ? sub * 8 : 0, p.rot, cs, sn, act, it.rc);
 }
 
 // nwg_to_signal > 0 (fused kernel): a completed head counts towards the kBarHeads event of that many workgroups.
-template <bool PAGED = false>
+template <bool PAGED = false, bool PAIRS = false>
 __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& it, int lane, int nwg_to_signal, int tag) {
     const int grp = lane >> 4, sub = lane & 15;
     const int D = p.D, H = p.H;
@@ -790,7 +803,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
 
     const RopeCoeffs& rc = it.rc;
     float q[8];
-    rope_load8(raw, d0, p.rot, rc, act, q);
+    rope_load8<PAIRS>(raw, d0, p.rot, rc, act, q);
 #pragma unroll
     for (int j = 0; j < 8; ++j) q[j] *= p.qscale;
 
@@ -801,7 +814,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     // the new token: split 0 owns it (appends it, returns it, and seeds its softmax state with it)
     if (sp == 0 && grp == 0) {
         float kf[8], vf[8];
-        rope_load8(raw + p.qkv_k_off, d0, p.rot, rc, act, kf);
+        rope_load8<PAIRS>(raw + p.qkv_k_off, d0, p.rot, rc, act, kf);
         raw_load8(raw + p.qkv_v_off, d0, act, vf);
         const u32x4 kp = pack8(kf), vp = pack8(vf);
         unpack8(kp, kf); unpack8(vp, vf);      // attend over the fp16 values the cache will hold

@@ -785,7 +785,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     }
 }
 
-// Fused add + RMSNorm of the input rows, one wave per sequence: y = fp16(r * rstd * w), r = fp16(x + x_add) -> sum_out.
+// (Fused add +) RMSNorm of the input rows, one wave per sequence: y = fp16(r * rstd * w), r = fp16(x + x_add) -> sum_out
+// (r = x without x_add).
 struct BatchNorm {
     const half_t *x, *x_add, *norm_w;
     half_t *sum_out, *y;
@@ -811,14 +812,18 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_norm(BatchNorm a) {
         const int col = i * kChunk + lane * 8;
         const bool in = col < a.K;
         u32x4 r = {0u, 0u, 0u, 0u}, ra = {0u, 0u, 0u, 0u};
-        if (in) { r = ld16(a.x + base + col); ra = ld16(a.x_add + base + col); }
-        float w[8];
-        unpack8(r, v[i]); unpack8(ra, w);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[i][j] += w[j];
-        r = pack8(v[i]);
+        if (in) r = ld16(a.x + base + col);
         unpack8(r, v[i]);
-        if (in) *reinterpret_cast<u32x4*>(a.sum_out + base + col) = r;
+        if (a.x_add != nullptr) {
+            if (in) ra = ld16(a.x_add + base + col);
+            float w[8];
+            unpack8(ra, w);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[i][j] += w[j];
+            r = pack8(v[i]);
+            unpack8(r, v[i]);
+            if (in) *reinterpret_cast<u32x4*>(a.sum_out + base + col) = r;
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) ss += v[i][j] * v[i][j];
     }
@@ -833,6 +838,98 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_norm(BatchNorm a) {
             for (int j = 0; j < 8; ++j) v[i][j] = v[i][j] * rstd * g[j];
             *reinterpret_cast<u32x4*>(a.y + base + col) = pack8(v[i]);
         }
+    }
+}
+
+// ---- products with weights stored [in, out] ---------------------------------------------------------------
+// y[o] = sum_k x[k] W[k][o] for `nsec` matrices stacked along k (W row s K + k belongs to matrix s; the outputs of
+// matrix s go to y[s O ..]): the layout of the reference's plain llama_decoder_layer op (reference
+// include/5090/llama/llama_kernel_dispatch.cu:44-58: tensor map with the output features innermost).  A workgroup
+// owns a panel of 512 output columns and a slice of the k range: every load instruction of a wave fetches 1 KB of
+// one weight row, lane l accumulates its eight columns with the row's x[k] (broadcast from the lane that holds it).
+// The slices of a panel meet in a scratch buffer; the workgroup that delivers the last one adds them up in slice
+// order (fixed order: the result does not depend on timing).
+struct GemvT {
+    const half_t* W; int K, O, nsec;
+    const half_t* x;                 // [K] fp16
+    float* part;                     // [panels][slices][512]
+    int* cnt;                        // [panels], zero between launches
+    float* out_f32; half_t* out_f16; // [nsec O], one of the two
+    int slices;                      // k slices per panel
+};
+__global__ __launch_bounds__(kStreamers * 64) void k_gemv_t(GemvT a) {
+    __shared__ float red[kStreamers][kChunk];
+    __shared__ int last_flag;
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int ppm = (a.O + kChunk - 1) / kChunk;            // panels per matrix
+    const int panels = a.nsec * ppm;
+    const int panel = blockIdx.x % panels, slice = blockIdx.x / panels;
+    if (slice >= a.slices) return;
+    const int sec = panel / ppm, col = (panel - sec * ppm) * kChunk + lane * 8;
+    const bool in = col < a.O;
+    // this wave's rows: slice `slice` of K, quarter `wave` of the slice
+    const int part_id = slice * kStreamers + wave, nparts = a.slices * kStreamers;
+    const int k0 = (int)(((long long)part_id * a.K) / nparts), k1 = (int)(((long long)(part_id + 1) * a.K) / nparts);
+    const half_t* wp = a.W + ((size_t)sec * a.K) * a.O + (in ? col : 0);
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    constexpr int kRows = 8;           // rows requested together
+    for (int kb = k0; kb < k1; kb += 64) {
+        const int n = k1 - kb < 64 ? k1 - kb : 64;
+        const float xv = lane < n ? (float)a.x[kb + lane] : 0.f;     // x[kb + lane]; rows past the range get 0
+        for (int r = 0; r < n; r += kRows) {
+            u32x4 w[kRows];
+#pragma unroll
+            for (int u = 0; u < kRows; ++u) {
+                const int k = kb + r + u < k1 ? kb + r + u : k1 - 1;
+                w[u] = ld_stream16(wp + (size_t)k * a.O);
+            }
+#pragma unroll
+            for (int u = 0; u < kRows; ++u) {
+                const float xk = rl(xv, r + u < 64 ? r + u : 63);    // 0 for rows past the range
+                float f[8];
+                unpack8(w[u], f);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[j] += xk * f[j];
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) red[wave][lane * 8 + j] = acc[j];
+    __syncthreads();
+    float* mine = a.part + ((size_t)panel * a.slices + slice) * kChunk;
+    for (int c = threadIdx.x; c < kChunk; c += kStreamers * 64) st_agent(mine + c, red[0][c] + red[1][c] + red[2][c] + red[3][c]);
+    drain_memory_ops();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int done = __hip_atomic_fetch_add(a.cnt + panel, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_flag = done == a.slices - 1;
+        if (last_flag) __hip_atomic_store(a.cnt + panel, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!last_flag) return;
+    const int pc0 = (panel - sec * ppm) * kChunk;
+    for (int c = threadIdx.x; c < kChunk; c += kStreamers * 64) {
+        if (pc0 + c >= a.O) continue;
+        float sum = 0.f;
+        for (int sl = 0; sl < a.slices; ++sl) sum += ld_agent(a.part + ((size_t)panel * a.slices + sl) * kChunk + c);
+        const size_t o = (size_t)sec * a.O + pc0 + c;
+        if (a.out_f32 != nullptr) a.out_f32[o] = sum;
+        else a.out_f16[o] = (half_t)sum;
+    }
+}
+
+// stage B with GPT-J pairing of the rotary dims
+__global__ __launch_bounds__(kStreamers * 64) void k_stage_b_pairs(LayerParams p) {
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int S = load_seq_len(p);
+    const int nsplit = effective_split(p, S);
+    const int item = blockIdx.x * kStreamers + wave;
+    if (item < p.heads * nsplit) {
+        AttnItem it;
+        attn_prefetch<false, true>(p, it, item / nsplit, item % nsplit, nsplit, S, lane);
+        attention_item<false, true>(p, it, lane, 0, 0);
     }
 }
 
@@ -1334,6 +1431,79 @@ int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_
     if (env_int("CFPP_LLAMA_SPLIT", 0) || p.heads > grid * kStreamers) return run_split(pl, p, a->seq_len, st);
     // one launch: the attention waves fetch their K/V tiles while the streaming waves do the QKV rows
     return launch_fused(pl, p, grid, st);
+}
+
+// The reference's plain llama_decoder_layer op: as cfpp_llama_attention_decode without a residual, with weights stored
+// [in, out] and GPT-J pairing of the rotary dims.  Four launches: norm, QKV products, attention items, O products.
+size_t cfpp_llama_plain_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim) {
+    const size_t base = cfpp_llama_workspace_bytes(hidden, heads, head_dim);
+    if (base == 0) return 0;
+    const int grid = streaming_grid();
+    const int ppm = (hidden + kChunk - 1) / kChunk;
+    const size_t units = (size_t)(3 * ppm > grid ? 3 * ppm : grid) + 3 * ppm;     // (panels x slices) never exceeds this
+    return base + align_up(units * kChunk * 4, 256) + align_up((size_t)3 * ppm * 4, 256) + align_up((size_t)hidden * 2, 256);
+}
+int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!a || !workspace) return CFPP_ERR_NULL;
+    const cfpp_neox_dims d = llama_dims(a->hidden, a->heads, a->head_dim, a->eps);
+    int rc = check_dims(&d);
+    if (rc) return rc;
+    const void* req[] = {a->rms_w, a->w_qkv, a->w_o, a->input, a->output, a->k_new, a->v_new, a->k_cache, a->v_cache, a->cos, a->sin};
+    for (const void* q : req) {
+        if (!q) return CFPP_ERR_NULL;
+        if (!aligned16(q)) return CFPP_ERR_ALIGN;
+    }
+    if (a->residual != nullptr || a->add_residual) return CFPP_ERR_MODE;      // this op has no residual stream
+    if (a->seq_len < 0) return CFPP_ERR_SEQ;
+    const size_t need = cfpp_llama_plain_workspace_bytes(a->hidden, a->heads, a->head_dim);
+    if (need == 0) return CFPP_ERR_DIMS;
+    if (workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CFPP_ERR_WORKSPACE;
+    const WorkspaceLayout L = workspace_layout(d);
+    Plan pl;
+    if ((rc = make_plan(d, &pl))) return rc;
+    if (!shape_supported(pl)) return CFPP_ERR_DIMS;
+    char* ws = reinterpret_cast<char*>(workspace);
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const int grid = streaming_grid();
+    const int H = d.hidden, ppm = (H + kChunk - 1) / kChunk;
+    const size_t units = (size_t)(3 * ppm > grid ? 3 * ppm : grid) + 3 * ppm;
+    float* part = reinterpret_cast<float*>(ws + L.total);
+    int* cnt = reinterpret_cast<int*>(ws + L.total + align_up(units * kChunk * 4, 256));
+    half_t* xn = reinterpret_cast<half_t*>(reinterpret_cast<char*>(cnt) + align_up((size_t)3 * ppm * 4, 256));
+    auto h = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
+
+    BatchNorm n{};
+    n.x = h(a->input); n.x_add = nullptr; n.norm_w = h(a->rms_w); n.sum_out = nullptr; n.y = xn;
+    n.eps = a->eps; n.K = H; n.batch = 1;
+    if ((rc = launch_batch_norm(pl.nch, n, st))) return rc;
+
+    cfpp_neox_weights w{};
+    w.ln_w = a->rms_w; w.ln_b = a->rms_w; w.w_qkv = a->w_qkv; w.b_qkv = a->rms_w; w.w_o = a->w_o; w.b_o = a->rms_w;
+    w.post_ln_w = a->rms_w; w.post_ln_b = a->rms_w; w.w_up = a->w_qkv; w.b_up = a->rms_w; w.w_down = a->w_qkv; w.b_down = a->rms_w;
+    cfpp_neox_io io{};
+    io.input = a->input; io.output = a->output; io.k_new = a->k_new; io.v_new = a->v_new;
+    io.k_cache = const_cast<void*>(a->k_cache); io.v_cache = const_cast<void*>(a->v_cache);
+    io.cache_rows = a->seq_len; io.cos = a->cos; io.sin = a->sin; io.rope_stride = 0; io.seq_len = a->seq_len;
+    LayerParams p;
+    if ((rc = fill_params(&d, &w, &io, workspace, workspace_bytes, true, true, &p, &pl))) return rc;
+    p.F = 0;
+    p.qkv_head_stride = d.head_dim; p.qkv_k_off = H; p.qkv_v_off = 2 * H;
+    p.append_kv = 0;
+
+    auto gemv = [&](const half_t* W, int nsec, const half_t* x, float* out_f32, half_t* out_f16) {
+        GemvT g{};
+        g.W = W; g.K = H; g.O = H; g.nsec = nsec; g.x = x; g.part = part; g.cnt = cnt;
+        g.out_f32 = out_f32; g.out_f16 = out_f16;
+        const int panels = nsec * ppm;
+        g.slices = grid / panels < 1 ? 1 : (grid / panels > 64 ? 64 : grid / panels);
+        hipLaunchKernelGGL(k_gemv_t, dim3(panels * g.slices), dim3(kStreamers * 64), 0, st, g);
+        return (int)hipGetLastError();
+    };
+    if ((rc = gemv(h(a->w_qkv), 3, xn, p.qkv_raw, nullptr))) return rc;
+    const int bgrid = (p.heads * split_bound(a->seq_len, p.max_split) + kStreamers - 1) / kStreamers;
+    hipLaunchKernelGGL(k_stage_b_pairs, dim3(bgrid), dim3(kStreamers * 64), 0, st, p);
+    if ((rc = (int)hipGetLastError())) return rc;
+    return gemv(h(a->w_o), 1, p.attn_vec, nullptr, reinterpret_cast<half_t*>(a->output));
 }
 
 size_t cfpp_llama_mlp_workspace_bytes(int32_t hidden, int32_t ffn) {

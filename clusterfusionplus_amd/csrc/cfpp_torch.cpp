@@ -446,6 +446,62 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> llama_decoder_layer_sglang(Tensor inp
     return std::make_tuple(std::get<0>(r), residual, std::get<1>(r), std::get<2>(r));
 }
 
+// llama_decoder_layer of the reference (include/pybind.cpp:66-75,280): (input, weight_qkv, weight_o, k_cache, v_cache,
+// rms_input_weight, cos, sin) -> (output, k, v).  Weights are stored [in, out] (weight_qkv = three such matrices
+// stacked), the rotary dims pair up GPT-J style, cos / sin hold head_dim entries, eps is 1e-6
+// (include/5090/llama/kernel.cuh:58), the caches are read only.
+std::tuple<Tensor, Tensor, Tensor> llama_decoder_layer(Tensor input, Tensor weight_qkv, Tensor weight_o, Tensor k_cache,
+                                                       Tensor v_cache, Tensor rms_input_weight, Tensor cos, Tensor sin,
+                                                       int64_t num_heads) {
+    const char* op = "llama_decoder_layer";
+    TORCH_CHECK(input.defined() && input.dim() >= 1, "input is undefined");
+    const int64_t H = input.numel();
+    TORCH_CHECK(num_heads > 0 && H % num_heads == 0, "hidden size ", H, " is not a multiple of num_heads ", num_heads);
+    const int64_t D = H / num_heads;
+    check_half(input, "input", H, input);
+    check_half(weight_qkv, "weight_qkv", 3 * H * H, input);
+    check_half(weight_o, "weight_o", H * H, input);
+    check_half(rms_input_weight, "rms_input_weight", H, input);
+    const int64_t rows_k = check_cache(k_cache, "k_cache", H, input);
+    const int64_t rows_v = check_cache(v_cache, "v_cache", H, input);
+    TORCH_CHECK(rows_k == rows_v, "k_cache has ", rows_k, " rows but v_cache has ", rows_v);
+    check_rope(cos, "cos", D, input);
+    check_rope(sin, "sin", D, input);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+    auto opts = input.options();
+    Tensor out = torch::empty({1, H}, opts);
+    Tensor k = torch::empty({1, num_heads, D}, opts);
+    Tensor v = torch::empty({1, num_heads, D}, opts);
+    cfpp_llama_attn a{};
+    a.hidden = (int32_t)H; a.heads = (int32_t)num_heads; a.head_dim = (int32_t)D; a.eps = 1e-6f;
+    a.rms_w = rms_input_weight.data_ptr(); a.w_qkv = weight_qkv.data_ptr(); a.w_o = weight_o.data_ptr();
+    a.input = input.data_ptr(); a.residual = nullptr; a.output = out.data_ptr(); a.add_residual = 0;
+    a.k_new = k.data_ptr(); a.v_new = v.data_ptr();
+    a.k_cache = rows_k > 0 ? k_cache.data_ptr() : input.data_ptr();
+    a.v_cache = rows_k > 0 ? v_cache.data_ptr() : input.data_ptr();
+    a.seq_len = (int32_t)rows_k;
+    a.cos = cos.data_ptr<float>(); a.sin = sin.data_ptr<float>();
+    const size_t bytes = cfpp_llama_plain_workspace_bytes(a.hidden, a.heads, a.head_dim);
+    TORCH_CHECK(bytes > 0, "unsupported layer dimensions (hidden ", H, ", heads ", num_heads, ")");
+    hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    static std::mutex mu;
+    static std::map<std::tuple<int, void*, int, int>, Tensor> cache;
+    Tensor ws;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto key = std::make_tuple((int)input.device().index(), (void*)st, (int)H, (int)D);
+        auto it = cache.find(key);
+        if (it == cache.end()) {
+            ws = torch::zeros({(int64_t)bytes + 256}, torch::TensorOptions().dtype(torch::kUInt8).device(input.device()));
+            cache[key] = ws;
+        } else {
+            ws = it->second;
+        }
+    }
+    check_rc(cfpp_llama_attention_plain(&a, ws_ptr(ws), bytes, st), op);
+    return std::make_tuple(out, k, v);
+}
+
 // llama_decoder_layer_batch_decode_sglang of the reference (include/pybind.cpp:90-106,282;
 // include/5090/llama/llama_kernel_batch_sglang_dispatch.cu:6-110): same positional arguments, results written into the
 // caller's `output` and `residual_output`, the new K/V rows into the paged caches; returns None.  The reference reads
@@ -570,6 +626,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("llama_decoder_layer_sglang", &llama_decoder_layer_sglang, py::arg("input"), py::arg("residual"), py::arg("weight_qkv"),
           py::arg("weight_o"), py::arg("k_cache"), py::arg("v_cache"), py::arg("rms_input_weight"), py::arg("eps"), py::arg("cos"),
           py::arg("sin"), py::arg("num_heads") = 32);
+    m.def("llama_decoder_layer", &llama_decoder_layer, py::arg("input"), py::arg("weight_qkv"), py::arg("weight_o"), py::arg("k_cache"),
+          py::arg("v_cache"), py::arg("rms_input_weight"), py::arg("cos"), py::arg("sin"), py::arg("num_heads") = 32);
     m.def("llama_decoder_layer_batch_decode_sglang", &llama_decoder_layer_batch_decode_sglang, py::arg("output"),
           py::arg("residual_output"), py::arg("input"), py::arg("residual"), py::arg("weight_qkv"), py::arg("weight_o"),
           py::arg("paged_kv_indptr"), py::arg("paged_kv_indices"), py::arg("k_cache_ptrs"), py::arg("v_cache_ptrs"),

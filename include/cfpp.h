@@ -138,6 +138,15 @@ typedef struct cfpp_llama_attn {
 size_t cfpp_llama_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim);
 int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The reference's plain op (llama_decoder_layer_sm120, reference include/pybind.cpp:66-75,280;
+ * include/5090/llama/llama_kernel_dispatch.cu:4-145): output = W_o^T attn, no residual stream (residual must be NULL,
+ * add_residual 0), weights stored [in, out]: w_qkv is [3H, H] = three [H_in, H_out] matrices for q, k, v stacked,
+ * w_o is [H_in, H_out]; GPT-J pairing of the rotary dims (dim 2i with 2i+1; include/5090/llama/kernel.cuh:298-314)
+ * with cos / sin tables of head_dim entries indexed by the dim (:280-281).  Caches are not written.
+ * Workspace: cfpp_llama_plain_workspace_bytes, 256-byte aligned, zero-initialised once, one per stream. */
+size_t cfpp_llama_plain_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim);
+int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- LLaMA MLP block ---------------------------------------------------------------------------------
  * output = input + W_down (silu(Wg n) * (Wu n)),  n = RMSNorm(input; eps) * rms_w,  w_gate_up = [Wg; Wu] ([2F, H]),
  * w_down [H, F].  Two launches (norm + gated up rows, down rows + residual).  The reference fuses only the

@@ -311,6 +311,48 @@ def llama_attention_sglang(
     return {"output": out, "residual": r, "k_new": k_new[None], "v_new": v_new[None], "attn_heads": o}
 
 
+def rope_pairs_gptj(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """GPT-J RoPE over the whole last dim: dims (2i, 2i+1) rotate together, tables indexed by the dim
+    (reference include/5090/llama/kernel.cuh:280-281,298-314; tests/test_llama.py:31-36,48-51):
+    out[2i] = t[2i] cos[2i] - t[2i+1] sin[2i],  out[2i+1] = t[2i+1] cos[2i+1] + t[2i] sin[2i+1]."""
+    D = t.shape[-1]
+    cos = cos.reshape(-1)[:D].to(t.dtype)
+    sin = sin.reshape(-1)[:D].to(t.dtype)
+    partner = torch.stack((-t[..., 1::2], t[..., 0::2]), dim=-1).reshape(t.shape)
+    return t * cos + partner * sin
+
+
+def llama_attention_plain(
+    x: torch.Tensor,
+    w: Dict[str, torch.Tensor],
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    cos: torch.Tensor,
+    sin: torch.Tensor,
+    dims: LlamaDims,
+    dtype: torch.dtype = torch.float32,
+    round_io: bool = True,
+) -> Dict[str, torch.Tensor]:
+    """The reference's plain `llama_decoder_layer` op (include/5090/llama/kernel.cuh): RMSNorm (eps 1e-6, :58,131),
+    q/k/v = n @ W with weights stored [in, out] (`w_qkv_t` [3H, H]: three such matrices stacked,
+    llama_kernel_dispatch.cu:44-58; kernel.cuh:144,187,230), GPT-J RoPE on q and k (:298-314), attention over every
+    cache row plus the new token, output = attn @ `w_o_t` ([in, out], :573), no residual, caches not written."""
+    H, nh, D = dims.hidden, dims.heads, dims.head_dim
+    f = lambda t: t.detach().to("cpu").to(dtype)
+    n1 = rms_norm(f(x).reshape(1, H), f(w["rms1"]).reshape(H), 1e-6)
+    wq, wk, wv = f(w["w_qkv_t"]).reshape(3, H, H)
+    q = rope_pairs_gptj((n1 @ wq).reshape(nh, D), f(cos), f(sin))
+    k_new = _r16(rope_pairs_gptj((n1 @ wk).reshape(nh, D), f(cos), f(sin)), round_io)
+    v_new = _r16((n1 @ wv).reshape(nh, D), round_io)
+    S = k_cache.shape[0]
+    keys = torch.cat([f(k_cache).reshape(S, nh, D), k_new[None]], dim=0).permute(1, 0, 2)
+    vals = torch.cat([f(v_cache).reshape(S, nh, D), v_new[None]], dim=0).permute(1, 0, 2)
+    pr = torch.softmax(torch.einsum("hd,hsd->hs", q, keys) / math.sqrt(D), dim=-1)
+    o = torch.einsum("hs,hsd->hd", pr, vals)
+    out = _r16(o.reshape(1, H) @ f(w["w_o_t"]), round_io)
+    return {"output": out, "k_new": k_new[None], "v_new": v_new[None], "attn_heads": o}
+
+
 def llama_batch_decode_paged(
     x: torch.Tensor,
     residual: torch.Tensor,

@@ -316,3 +316,46 @@ def test_llama_batch_decode_paged_matches_hf_per_sequence():
     keep = torch.ones(pool, dtype=torch.bool)
     keep[touched] = False
     assert torch.equal(got["k_cache"][keep], k[keep]) and torch.equal(got["v_cache"][keep], v[keep])
+
+
+def test_rope_pairs_gptj_matches_hf_gptj_rotary():
+    """Pairing and sign convention of the GPT-J rotary, against HF's GPT-J helper (tables with one angle per pair,
+    repeated for the two dims of the pair, as `apply_rotary_pos_emb` of modeling_gptj builds them)."""
+    hf = pytest.importorskip("transformers")
+    from transformers.models.gptj.modeling_gptj import apply_rotary_pos_emb as gptj_rope
+    g = torch.Generator().manual_seed(3)
+    D = 16
+    t = torch.randn(1, 1, 4, D, generator=g, dtype=torch.float64)        # [batch, seq, heads, dim]
+    ang = torch.rand(D // 2, generator=g, dtype=torch.float64) * 6.28
+    sin_h, cos_h = torch.sin(ang)[None, None, :], torch.cos(ang)[None, None, :]       # HF repeats each entry twice itself
+    want = gptj_rope(t, sin_h, cos_h)
+    cos = torch.repeat_interleave(torch.cos(ang), 2)
+    sin = torch.repeat_interleave(torch.sin(ang), 2)
+    got = O.rope_pairs_gptj(t[0, 0], cos, sin)
+    assert torch.allclose(got, want[0, 0], atol=1e-12, rtol=0)
+    # a rotation of each pair: norms of the pairs are kept, angle 0 is the identity
+    assert torch.allclose(got.reshape(4, D // 2, 2).norm(dim=-1), t[0, 0].reshape(4, D // 2, 2).norm(dim=-1), atol=1e-12)
+    assert torch.equal(O.rope_pairs_gptj(t[0, 0], torch.ones(D, dtype=torch.float64), torch.zeros(D, dtype=torch.float64)), t[0, 0])
+
+
+def test_llama_attention_plain_is_the_sglang_block_with_transposed_weights_and_gptj_pairs():
+    """With zero angles both ops apply no rotation: the plain op on transposed weights must equal the (HF-pinned)
+    sglang block without a residual; with angles, q and k of the plain op are the GPT-J rotation of the unrotated ones."""
+    dims, S, w, x, res, k, v, cos, sin = _tiny_llama()
+    H, D = dims.hidden, dims.head_dim
+    wt = {"rms1": w["rms1"], "w_qkv_t": w["w_qkv"].reshape(3, H, H).transpose(1, 2).contiguous().reshape(3 * H, H),
+          "w_o_t": w["w_o"].t().contiguous()}
+    one, zero = torch.ones(1, D), torch.zeros(1, D)
+    a = O.llama_attention_plain(x, wt, k, v, one, zero, dims, dtype=torch.float64, round_io=False)
+    b = O.llama_attention_sglang(x, None, w, k, v, one, zero, dims, dtype=torch.float64, round_io=False)
+    assert torch.allclose(a["output"], b["output"], atol=1e-12, rtol=0)
+    assert torch.allclose(a["k_new"], b["k_new"], atol=1e-12, rtol=0) and torch.allclose(a["v_new"], b["v_new"], atol=1e-12, rtol=0)
+    g = torch.Generator().manual_seed(9)
+    ang = torch.rand(D // 2, generator=g, dtype=torch.float64) * 6.28
+    c2, s2 = torch.repeat_interleave(torch.cos(ang), 2), torch.repeat_interleave(torch.sin(ang), 2)
+    r = O.llama_attention_plain(x, wt, k, v, c2, s2, dims, dtype=torch.float64, round_io=False)
+    assert torch.allclose(r["k_new"][0], O.rope_pairs_gptj(a["k_new"][0], c2, s2), atol=1e-12, rtol=0)
+    assert torch.equal(r["v_new"], a["v_new"])
+    # S = 0: the only key is the new token
+    r0 = O.llama_attention_plain(x, wt, k[:0], v[:0], c2, s2, dims, dtype=torch.float64, round_io=False)
+    assert torch.allclose(r0["attn_heads"], r0["v_new"][0], atol=1e-12, rtol=0)
