@@ -236,6 +236,7 @@ struct FusedLds {
     LnShared<NCH> lns;
     float park_mem[kStreamers][kParkRows];
     int park_rows[kStreamers][kParkRows];
+    float park_attn[kStreamers][kParkRows];   // QKV rows of the attention waves
 };
 
 // One layer; `gen` is the launch generation read at the start of the launch.
@@ -260,14 +261,23 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
     // wave, so that it is on its way while the statistics are computed
     constexpr int kFusedWaves = 2 * kStreamers;
     constexpr int RPIA = StageARpi<NCH>::value;
-    const RowWalk qw = row_walk<RPIA>(false, b * kStreamers + wave, nsw, 0, 3 * p.H);     // streaming waves only
+    // QKV rows: shared by all eight waves of every workgroup (the attention waves have nothing else to do until the
+    // QKV rows exist, and twice as many loads in flight stream faster), or by the streaming waves only
+    // (only when that leaves every wave three tiles or more: with fewer, the attention waves start their items later
+    // than the shorter QKV pass gains)
+    const int qkv_units = (3 * p.H + RPIA - 1) / RPIA;
+    const bool qkv8 = p.qkv_all_waves > 0 || (p.qkv_all_waves < 0 && qkv_units >= 3 * G * kFusedWaves);
+    const RowWalk qw = qkv8 ? row_walk<RPIA>(false, b * kFusedWaves + wave, G * kFusedWaves, 0, 3 * p.H)
+                            : row_walk<RPIA>(false, b * kStreamers + (wave < kStreamers ? wave : 0), nsw, 0,
+                                             wave < kStreamers ? 3 * p.H : 0);
+    const int qkv_arrivals = qkv8 ? kFusedWaves : kStreamers;
     const int hw = wave - kStreamers;
     RowTile<NCH, RPIA> t0;
     {
         LnOwn<NCH, kFusedWaves> own;
         ln_coop_load<NCH, kFusedWaves, true>(own, norm_spec(p), wave, lane);
         __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
-        if (wave < kStreamers) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
+        if (qkv8 || wave < kStreamers) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
         ln_coop_finish<NCH, kFusedWaves, true>(own, norm_spec(p), lns, wave, lane);
     }
     const int tag = first_lane(gen) + 1;
@@ -318,7 +328,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
         if (dynamic) {
             TeamTiles<NCH, kUpRpi> ut;
             team_prefetch<NCH, kUpRpi, EX>(p.w_up, p.H, utm, lane, ut);
-            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], kStreamers, tag);
+            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
             trace_mark(p, 2);
             ln_fetch<NCH>(lns, 1, lane, xr);
 #pragma unroll
@@ -335,7 +345,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
             RowTile<NCH, kUpRpi> u0;
             RowWalk uw = row_walk<kUpRpi>(false, b * kStreamers + wave, nsw, 0, up_phase_rows(CPD, 0, p.F));
             up_prefetch<NCH, EX>(p, uw, lane, u0);
-            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], kStreamers, tag);
+            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
             trace_mark(p, 2);
             ln_fetch<NCH>(lns, 1, lane, xr);
 #pragma unroll
@@ -353,6 +363,13 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
         // an attention wave takes the (head, split) item b + hw G (the host caps the KV splits so that no wave has
         // more than one item: attn_count <= kStreamers); what does not depend on the QKV rows (first K/V tiles,
         // RoPE coefficients) is requested before waiting for them
+        if (qkv8) {
+            RowPark hpark{lds.park_attn[hw], 0};
+            half2_t xq[NCH][4];
+            ln_fetch<NCH>(lns, 0, lane, xq);
+            qkv_rows<NCH, EX>(p, xq, qw, lane, t0, hpark);
+            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
+        }
         if (hw < attn_count) {
             AttnItem it;
             attn_prefetch(p, it, (b + hw * G) / nsplit, (b + hw * G) % nsplit, nsplit, S, lane);
@@ -1219,6 +1236,7 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     p.append_kv = 1; p.x_add = nullptr; p.x_sum_out = nullptr; p.c_add_sum = 0;
     p.dyn_up = env_int("CFPP_DYN_UP", -1);
     p.arrival_agents = env_int("CFPP_ARRIVAL_AGENTS", 1);
+    p.qkv_all_waves = env_int("CFPP_QKV_ALL_WAVES", -1);   // -1: decided by the geometry
     char* ws = reinterpret_cast<char*>(workspace);
     p.qkv_raw = reinterpret_cast<float*>(ws + L.qkv_raw);
     p.attn_vec = reinterpret_cast<half_t*>(ws + L.attn_vec);
