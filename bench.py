@@ -120,7 +120,7 @@ def cpu_baseline(cfg, S, budget_s=12.0):
     }
 
 
-def bench_llama_layer(args):
+def bench_llama_layer(args, emit=True):
     """Extra workload (not the headline): one LLaMA-2-7B layer, batch-1 decode at context --ctx (default 4096):
     the attention block (the reference's llama_decoder_layer_sglang) followed by the MLP block, replayed from a
     captured graph over 8 weight sets so that every launch reads HBM-cold weights."""
@@ -163,7 +163,7 @@ def bench_llama_layer(args):
     us = e0.elapsed_time(e1) * 1e3 / (reps * nset)
     nbytes = 2 * (3 * H * H + H * H + 3 * F * H) + 2 * 2 * H + S * 2 * H * 2
     gbps = nbytes / (us * 1e-6) / 1e9
-    print(json.dumps({
+    result = {
         "metric": "layer_latency_us", "value": round(us, 2), "unit": "us/layer", "n_gpus": 1, "steps": reps * nset, "warmup": args.warmup,
         "ms_per_step": round(us * 1e-3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
@@ -172,10 +172,13 @@ def bench_llama_layer(args):
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
                      "traffic": None, "kernel": "k_fused (attention block) + k_gated_up + k_stage_c", "bytes_per_launch": nbytes,
                      "launch_us": round(us, 2)},
-        "cpu_baseline": None}), flush=True)
+        "cpu_baseline": None}
+    if emit:
+        print(json.dumps(result), flush=True)
+    return result
 
 
-def bench_llama_batch(args):
+def bench_llama_batch(args, emit=True):
     """Extra workload (not the headline): the LLaMA-2-7B attention block for --batch sequences of --ctx cached tokens
     each over paged caches (the reference's llama_decoder_layer_batch_decode_sglang), pages scattered over the pool,
     six weight sets in turn so that every call reads HBM-cold weights."""
@@ -222,7 +225,7 @@ def bench_llama_batch(args):
     us = e0.elapsed_time(e1) * 1e3 / args.steps
     nbytes = 2 * 4 * H * H + 2 * H + B * S * 2 * H * 2
     gbps = nbytes / (us * 1e-6) / 1e9
-    print(json.dumps({
+    result = {
         "metric": "batch_step_latency_us", "value": round(us, 2), "unit": "us/call", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(us * 1e-3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
@@ -232,7 +235,66 @@ def bench_llama_batch(args):
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
                      "traffic": None, "kernel": "k_batch_norm + k_batch_mfma_lds (QKV) + k_batch_attn + k_batch_mfma_lds (O)",
                      "bytes_per_launch": nbytes, "launch_us": round(us, 2)},
-        "cpu_baseline": None}), flush=True)
+        "cpu_baseline": None}
+    if emit:
+        print(json.dumps(result), flush=True)
+    return result
+
+
+def other_workloads(pkg, dev, args):
+    """Short measurements of the other configurations, appended to the headline line (each is also a workload of its
+    own: --model pythia_2b8 / llama2_7b_layer / llama2_7b_batch).  A failure is reported, not raised."""
+    import copy
+    import torch
+    out = []
+
+    def attempt(name, fn):
+        try:
+            out.append(fn())
+        except Exception as e:     # noqa: BLE001
+            log(f"[other_workloads] {name} failed: {type(e).__name__}: {e}")
+            out.append({"workload": name, "error": f"{type(e).__name__}: {e}"})
+
+    def stack_2b8():
+        cfg, ctx, K, W = pkg.PYTHIA_2B8, 1024, 64, 8
+        dec = build_model(cfg, ctx + W + K + 40, ctx, dev, "fused")
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            dec.set_state(11, ctx)
+            dec.graph_steps(W)
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            dec.graph_steps(K)
+            e1.record(stream)
+            stream.synchronize()
+        tpot = e0.elapsed_time(e1) / K
+        sb = step_bytes(cfg, ctx + W + K // 2)
+        return {"workload": "pythia_2b8 full stack, batch-1 greedy decode, hipGraph replay, context 1024", "metric": "tpot_ms",
+                "value": round(tpot, 4), "unit": "ms/token", "bytes": sb, "hbm_gbps": round(sb / (tpot * 1e-3) / 1e9, 1),
+                "frac_of_peak": round(sb / (tpot * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+
+    def brief(r):
+        return {"workload": r["config"]["workload"], "metric": r["metric"], "value": r["value"], "unit": r["unit"],
+                "bytes": r["roofline"]["bytes_per_launch"], "hbm_gbps": r["roofline"]["achieved"], "frac_of_peak": r["roofline"]["frac"]}
+
+    def llama_layer():
+        a = copy.copy(args)
+        a.ctx, a.steps, a.warmup = 4096, 64, 8
+        return brief(bench_llama_layer(a, emit=False))
+
+    def llama_batch():
+        a = copy.copy(args)
+        a.ctx, a.batch, a.steps, a.warmup = 1024, 16, 60, 12
+        return brief(bench_llama_batch(a, emit=False))
+
+    attempt("pythia_2b8 full stack", stack_2b8)
+    torch.cuda.empty_cache()
+    attempt("llama2_7b decoder layer", llama_layer)
+    torch.cuda.empty_cache()
+    attempt("llama2_7b paged batch", llama_batch)
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -245,6 +307,7 @@ def main():
     ap.add_argument("--ctx", type=int, default=2048, help="KV-cache rows already filled when the timed region starts")
     ap.add_argument("--mode", default="fused", choices=["fused", "split"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-also", dest="also", action="store_false", help="skip the short measurements of the other configurations")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU (the hot path is a single-GPU batch-1 decode step); "
@@ -330,6 +393,10 @@ def main():
                  "roofline_ms": round(sb / (HBM_PEAK_GBPS * 1e9) * 1e3, 4), "event_ms_per_step": round(ev_ms / K, 4),
                  "lm_head_us": round(sorted(lm_ms)[1] * 1e3, 1)},
     }
+    if args.also and args.model == "pythia_6b9":
+        del dec
+        torch.cuda.empty_cache()
+        result["other_workloads"] = other_workloads(pkg, dev, args)
     if not args.no_cpu_baseline:
         try:
             result["cpu_baseline"] = cpu_baseline(cfg, args.ctx)
