@@ -70,6 +70,8 @@ struct LayerParams {
     int max_split;      // cap on the KV splits per head (<= kMaxSplit)
     int row_walk_strided;   // streaming waves take interleaved instead of contiguous row ranges
     const int* kv_rows;     // paged caches: cache row r of this sequence lives in row kv_rows[r] of k_cache / v_cache (null: r itself)
+    const int* tag_src;     // launch tags from a counter the caller advances between launches (null: from kBarGen)
+    int tag_mul, tag_add;   // tag = tag_src[0] * tag_mul + tag_add + 1
     int qkv_all_waves;      // fused kernel: the attention waves share the QKV rows with the streaming waves
     int arrival_agents;     // an idle attention wave carries the streaming waves' MLP-up arrivals to the device-wide counters
     int dyn_up;             // MLP-up tiles handed out dynamically within teams of workgroups: 1 yes, 0 no, -1 by size

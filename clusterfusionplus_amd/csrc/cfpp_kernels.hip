@@ -397,7 +397,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
     }
     trace_mark(p, 10);
     // the last workgroup to leave publishes the new generation: the flags of this launch turn stale
-    if (wave == 0) {
+    if (wave == 0 && p.tag_src == nullptr) {
         const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1, tag);
         if (last && lane == 0) __hip_atomic_store(p.bar + kBarGen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -407,8 +407,10 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
 template <int NCH, int CPD, bool EX>
 __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     __shared__ FusedLds<NCH> lds;
-    // the flag value of this launch is gen + 1: requested first, needed at the first event
-    const int gen = counter_peek(p.bar + kBarGen);
+    // the flag value of this launch is gen + 1: requested first, needed at the first event.  It comes from the
+    // generation the previous launch on this workspace published, or from a counter that the caller advances
+    // between launches (a whole-model step: step counter x layers + layer), which saves the publishing.
+    const int gen = p.tag_src != nullptr ? p.tag_src[0] * p.tag_mul + p.tag_add : counter_peek(p.bar + kBarGen);
     fused_layer<NCH, CPD, EX>(p, gen, lds);
 }
 
@@ -504,6 +506,7 @@ __global__ __launch_bounds__(256) void k_pick_and_advance(const float* __restric
         state[0] = bi;
         state[1] = state[1] + 1;
         state[2] = step + 1;
+        state[3] = state[3] + 1;      // steps since the stack was created: never reset, launch tags derive from it
         if (step < hist_cap) history[step] = bi;
     }
 }
@@ -1840,7 +1843,7 @@ struct cfpp_neox_stack {
     Plan plan{};
     int device = 0, grid = 0;
     char* slab = nullptr;
-    int* state = nullptr;         // {token, seq_len, step}
+    int* state = nullptr;         // {token, seq_len, step, steps since creation}
     half_t* hidden[2] = {nullptr, nullptr};
     half_t *k_new = nullptr, *v_new = nullptr;
     float* logits = nullptr;
@@ -1874,7 +1877,17 @@ cfpp_neox_io stack_layer_io(const cfpp_neox_stack* s, int l) {
 }
 int stack_enqueue_layer(cfpp_neox_stack* s, int l, hipStream_t st) {
     const cfpp_neox_io io = stack_layer_io(s, l);
-    return cfpp_neox_layer_decode(&s->desc.dims, &s->layers[l], &io, s->desc.mode, s->ws, s->ws_bytes, st);
+    if (s->desc.mode != CFPP_MODE_FUSED || !env_int("CFPP_STACK_TAGS", 1))
+        return cfpp_neox_layer_decode(&s->desc.dims, &s->layers[l], &io, s->desc.mode, s->ws, s->ws_bytes, st);
+    LayerParams p;
+    Plan pl;
+    int rc = fill_params(&s->desc.dims, &s->layers[l], &io, s->ws, s->ws_bytes, true, true, &p, &pl);
+    if (rc) return rc;
+    const int grid = fused_grid();
+    if (p.heads > grid * kStreamers) return run_split(pl, p, seq_hint_of(&io), st);
+    // launch tags from the stack's step counter: no launch has to publish a generation for the next one
+    p.tag_src = s->state + 3; p.tag_mul = s->desc.n_layers; p.tag_add = l;
+    return launch_fused(pl, p, grid, st);
 }
 
 int stack_enqueue_step(cfpp_neox_stack* s, hipStream_t st) {
