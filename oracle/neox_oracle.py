@@ -403,6 +403,42 @@ def make_llama_attn_inputs(dims: LlamaDims, S: int, seed: int = 0, w_std: float 
     return w, x, res, k, v, cos, sin
 
 
+def make_llama_plain_inputs(dims: LlamaDims, S: int, seed: int = 0, w_std: float = 0.02):
+    """Seeded fp16 tensors for the plain LLaMA op: weights dict (`rms1`, `w_qkv_t` [3H,H] = three [in,out] matrices,
+    `w_o_t` [in,out]), input [1,H], caches [S,H], cos/sin [1,D] with one random angle per (2i, 2i+1) pair."""
+    H, D = dims.hidden, dims.head_dim
+    g = torch.Generator().manual_seed(8200 + seed)
+    rn = lambda *shape, std=1.0: (torch.randn(*shape, generator=g) * std).half()
+    w = {"rms1": (1 + 0.1 * torch.randn(H, generator=g)).half(), "w_qkv_t": rn(3 * H, H, std=w_std), "w_o_t": rn(H, H, std=w_std)}
+    x, k, v = rn(1, H), rn(S, H), rn(S, H)
+    ang = torch.rand(1, D // 2, generator=g) * (2 * math.pi)
+    cos = torch.repeat_interleave(torch.cos(ang), 2, dim=-1).float().contiguous()
+    sin = torch.repeat_interleave(torch.sin(ang), 2, dim=-1).float().contiguous()
+    return w, x, k, v, cos, sin
+
+
+def make_llama_batch_inputs(dims: LlamaDims, lens, seed: int = 0, max_pos: int = 512, w_std: float = 0.02, layers: int = 3):
+    """Seeded inputs of the paged batch op: sequences of `lens` cached tokens each, their pages scattered over a shared
+    pool of cache rows (one pool per layer).  Returns (w, x [B,H], residual [B,H], indptr, indices, caches = [(k, v)] per
+    layer, positions, cos_sin [max_pos, D])."""
+    H, D, B = dims.hidden, dims.head_dim, len(lens)
+    g = torch.Generator().manual_seed(9100 + seed)
+    rn = lambda *shape, std=1.0: (torch.randn(*shape, generator=g) * std).half()
+    w = {"rms1": (1 + 0.1 * torch.randn(H, generator=g)).half(), "w_qkv": rn(3 * H, H, std=w_std), "w_o": rn(H, H, std=w_std)}
+    x, res = rn(B, H), rn(B, H)
+    total = sum(lens) + B
+    pool = total + 37
+    indices = torch.randperm(pool, generator=g)[:total].to(torch.int32)
+    indptr = torch.zeros(B + 1, dtype=torch.int32)
+    indptr[1:] = torch.cumsum(torch.tensor([n + 1 for n in lens]), 0).to(torch.int32)
+    caches = [(rn(pool, H), rn(pool, H)) for _ in range(layers)]
+    positions = torch.randint(0, max_pos, (B,), generator=g, dtype=torch.int64)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2).float() / D))
+    ang = torch.arange(max_pos).float()[:, None] * inv[None, :]
+    cos_sin = torch.cat([torch.cos(ang), torch.sin(ang)], dim=-1).float().contiguous()
+    return w, x, res, indptr, indices, caches, positions, cos_sin
+
+
 # --------------------------------------------------------------------------------------
 # Seeded synthetic inputs shared by tests, smoke and the benchmark
 # --------------------------------------------------------------------------------------

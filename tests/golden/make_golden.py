@@ -45,8 +45,45 @@ def llama_inputs(name):
     return (dims,) + tuple(O.make_llama_attn_inputs(dims, S, seed=seed))
 
 
+# plain LLaMA op (llama_attention_plain): dims, cache rows, seed
+LLAMA_PLAIN_CASES = {"llama_plain_h1024_s200": (O.LlamaDims(hidden=1024, heads=8, head_dim=128, ffn=0), 200, 3)}
+# paged batch (llama_batch_decode_paged): dims, cached tokens per sequence, seed, layer whose caches are used
+LLAMA_BATCH_CASES = {"llama_batch_h1024": (O.LlamaDims(hidden=1024, heads=8, head_dim=128, ffn=0), [77, 5, 300, 0, 41], 4, 1)}
+
+
+def llama_plain_inputs(name):
+    dims, S, seed = LLAMA_PLAIN_CASES[name]
+    return (dims,) + tuple(O.make_llama_plain_inputs(dims, S, seed=seed, w_std=0.05))
+
+
+def llama_batch_inputs(name):
+    dims, lens, seed, layer_id = LLAMA_BATCH_CASES[name]
+    return (dims, layer_id) + tuple(O.make_llama_batch_inputs(dims, lens, seed=seed, w_std=0.05))
+
+
+def new_rows(indptr, indices):
+    return [int(indices[int(indptr[b + 1]) - 1]) for b in range(indptr.numel() - 1)]
+
+
 def main():
     torch.set_num_threads(max(1, os.cpu_count() or 1))
+    for name in LLAMA_PLAIN_CASES:
+        dims, w, x, k, v, cos, sin = llama_plain_inputs(name)
+        r = O.llama_attention_plain(x, w, k, v, cos, sin, dims, dtype=torch.float64, round_io=True)
+        out = {n: r[n].to(torch.float32).numpy() for n in ("output", "k_new", "v_new")}
+        path = os.path.join(HERE, name + ".npz")
+        np.savez_compressed(path, **out)
+        print(name, {n: a.shape for n, a in out.items()}, os.path.getsize(path), "bytes")
+    for name in LLAMA_BATCH_CASES:
+        dims, layer_id, w, x, res, indptr, indices, caches, positions, cos_sin = llama_batch_inputs(name)
+        k, v = caches[layer_id]
+        r = O.llama_batch_decode_paged(x, res, w, indptr, indices, k, v, positions, cos_sin, dims, dtype=torch.float64)
+        rows = new_rows(indptr, indices)
+        out = {"output": r["output"].to(torch.float32).numpy(), "residual": r["residual"].to(torch.float32).numpy(),
+               "k_rows": r["k_cache"][rows].to(torch.float32).numpy(), "v_rows": r["v_cache"][rows].to(torch.float32).numpy()}
+        path = os.path.join(HERE, name + ".npz")
+        np.savez_compressed(path, **out)
+        print(name, {n: a.shape for n, a in out.items()}, os.path.getsize(path), "bytes")
     for name in LLAMA_CASES:
         dims, w, x, res, k, v, cos, sin = llama_inputs(name)
         r = O.llama_attention_sglang(x, res, w, k, v, cos, sin, dims, dtype=torch.float64, round_io=True)

@@ -88,3 +88,51 @@ def test_hip_matches_llama_golden(name):
     assert_close("k_new", k_new, want["k_new"])
     assert_close("v_new", v_new, want["v_new"])
     assert torch.equal(res_g.cpu().float().reshape(-1), want["residual"].reshape(-1))
+
+
+def test_oracle_reproduces_llama_plain_and_batch_golden():
+    dims, w, x, k, v, cos, sin = G.llama_plain_inputs("llama_plain_h1024_s200")
+    want = load("llama_plain_h1024_s200")
+    r = O.llama_attention_plain(x, w, k, v, cos, sin, dims, dtype=torch.float32)
+    for n in ("output", "k_new", "v_new"):
+        assert float((r[n].float() - want[n]).abs().max()) <= 8e-3, n
+        assert float((r[n].float() - want[n]).abs().mean()) <= 1e-4, n
+    dims, layer_id, w, x, res, indptr, indices, caches, positions, cos_sin = G.llama_batch_inputs("llama_batch_h1024")
+    want = load("llama_batch_h1024")
+    r = O.llama_batch_decode_paged(x, res, w, indptr, indices, caches[layer_id][0], caches[layer_id][1], positions, cos_sin, dims)
+    rows = G.new_rows(indptr, indices)
+    assert torch.equal(r["residual"].float(), want["residual"])
+    for got, n in ((r["output"], "output"), (r["k_cache"][rows], "k_rows"), (r["v_cache"][rows], "v_rows")):
+        assert float((got.float() - want[n]).abs().max()) <= 8e-3, n
+        assert float((got.float() - want[n]).abs().mean()) <= 1e-4, n
+
+
+@pytest.mark.gpu
+def test_hip_matches_llama_plain_and_batch_golden():
+    import clusterfusion as cf
+    from tests.test_gpu_layer_parity import assert_close
+    print("\ncase golden llama_plain_h1024_s200 / llama_batch_h1024", flush=True)
+    dev = "cuda:0"
+    dims, w, x, k, v, cos, sin = G.llama_plain_inputs("llama_plain_h1024_s200")
+    out, kn, vn = cf.llama_decoder_layer(x.to(dev), w["w_qkv_t"].to(dev), w["w_o_t"].to(dev), k.to(dev), v.to(dev), w["rms1"].to(dev),
+                                         cos.to(dev), sin.to(dev), num_heads=dims.heads)
+    torch.cuda.synchronize()
+    want = load("llama_plain_h1024_s200")
+    assert_close("output", out, want["output"])
+    assert_close("k_new", kn, want["k_new"])
+    assert_close("v_new", vn, want["v_new"])
+    dims, layer_id, w, x, res, indptr, indices, caches, positions, cos_sin = G.llama_batch_inputs("llama_batch_h1024")
+    gc = [(a.to(dev), b.to(dev)) for a, b in caches]
+    kptr = torch.tensor([a.data_ptr() for a, _ in gc], dtype=torch.uint64, device=dev)
+    vptr = torch.tensor([b.data_ptr() for _, b in gc], dtype=torch.uint64, device=dev)
+    out, res_out = torch.empty_like(x, device=dev), torch.empty_like(x, device=dev)
+    cf.llama_decoder_layer_batch_decode_sglang(out, res_out, x.to(dev), res.to(dev), w["w_qkv"].to(dev), w["w_o"].to(dev), indptr.to(dev),
+                                               indices.to(dev), kptr, vptr, layer_id, w["rms1"].to(dev), dims.eps, positions.to(dev),
+                                               cos_sin.to(dev))
+    torch.cuda.synchronize()
+    want = load("llama_batch_h1024")
+    rows = G.new_rows(indptr, indices)
+    assert_close("output", out, want["output"])
+    assert torch.equal(res_out.cpu().float(), want["residual"])
+    assert_close("k rows", gc[layer_id][0][rows], want["k_rows"])
+    assert_close("v rows", gc[layer_id][1][rows], want["v_rows"])

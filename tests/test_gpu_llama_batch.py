@@ -21,22 +21,7 @@ def cf():
 
 def make_case(dims, lens, seed, max_pos=512, w_std=0.02, layers=3, layer_id=1):
     """Sequences of `lens` cached tokens each; their pages are scattered over a shared pool of cache rows."""
-    H, D, B = dims.hidden, dims.head_dim, len(lens)
-    g = torch.Generator().manual_seed(9100 + seed)
-    rn = lambda *shape, std=1.0: (torch.randn(*shape, generator=g) * std).half()
-    w = {"rms1": (1 + 0.1 * torch.randn(H, generator=g)).half(), "w_qkv": rn(3 * H, H, std=w_std), "w_o": rn(H, H, std=w_std)}
-    x, res = rn(B, H), rn(B, H)
-    total = sum(lens) + B
-    pool = total + 37
-    perm = torch.randperm(pool, generator=g)[:total].to(torch.int32)
-    indptr = torch.zeros(B + 1, dtype=torch.int32)
-    indptr[1:] = torch.cumsum(torch.tensor([n + 1 for n in lens]), 0).to(torch.int32)
-    caches = [(rn(pool, H), rn(pool, H)) for _ in range(layers)]
-    positions = torch.randint(0, max_pos, (B,), generator=g, dtype=torch.int64)
-    inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2).float() / D))
-    ang = torch.arange(max_pos).float()[:, None] * inv[None, :]
-    cos_sin = torch.cat([torch.cos(ang), torch.sin(ang)], dim=-1).float().contiguous()
-    return w, x, res, indptr, perm, caches, positions, cos_sin, layer_id
+    return O.make_llama_batch_inputs(dims, lens, seed=seed, max_pos=max_pos, w_std=w_std, layers=layers) + (layer_id,)
 
 
 def run(cf, dims, lens, seed, **kw):

@@ -20,15 +20,7 @@ def cf():
 
 
 def make(dims, S, seed, w_std=0.02):
-    H, D = dims.hidden, dims.head_dim
-    g = torch.Generator().manual_seed(8200 + seed)
-    rn = lambda *shape, std=1.0: (torch.randn(*shape, generator=g) * std).half()
-    w = {"rms1": (1 + 0.1 * torch.randn(H, generator=g)).half(), "w_qkv_t": rn(3 * H, H, std=w_std), "w_o_t": rn(H, H, std=w_std)}
-    x, k, v = rn(1, H), rn(S, H), rn(S, H)
-    ang = torch.rand(1, D // 2, generator=g) * (2 * math.pi)
-    cos = torch.repeat_interleave(torch.cos(ang), 2, dim=-1).float().contiguous()      # one angle per (2i, 2i+1) pair
-    sin = torch.repeat_interleave(torch.sin(ang), 2, dim=-1).float().contiguous()
-    return w, x, k, v, cos, sin
+    return O.make_llama_plain_inputs(dims, S, seed=seed, w_std=w_std)
 
 
 def run(cf, dims, S, seed, **kw):
