@@ -233,7 +233,7 @@ def bench_llama_batch(args, emit=True):
                                "scattered), 4 launches per call", "batch": B, "context": S, "hidden": H,
                    "tokens_per_s_per_layer": round(B / (us * 1e-6))},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": None, "kernel": "k_batch_norm + k_batch_mfma_lds (QKV) + k_batch_attn + k_batch_mfma_lds (O)",
+                     "traffic": None, "kernel": "k_batch_norm + k_batch_mfma_pipe (QKV) + k_batch_attn + k_batch_mfma_pipe (O)",
                      "bytes_per_launch": nbytes, "launch_us": round(us, 2)},
         "cpu_baseline": None}
     if emit:

@@ -738,71 +738,84 @@ __global__ __launch_bounds__(512) void k_batch_mfma(BatchMfma a) {
     }
 }
 
-// Variant for row lengths that are multiples of 2048: the weights are requested row by row (a load instruction
-// fetches 1 KB of one row, as the row-streaming kernels do; the operand layout above makes an instruction fetch
-// 64 bytes from each of 16 rows, which the memory system serves at about two thirds of the rate) and take the
-// operand layout on their way through LDS: a wave writes 16 rows x 256 halfs at a time (rows padded by 16 bytes, so
-// that the sixteen rows a read touches fall into different banks) and reads the 16 x 32 blocks back.  Four waves per
-// workgroup, each with CH chunks of 512 halfs per row, all requested at once.
-constexpr int kMfmaRowBytes = kChunk + 16;      // half a chunk (256 halfs) per row at a time: three workgroups fit a compute unit
-template <int CH>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void k_batch_mfma_lds(BatchMfma a) {
-    __shared__ __attribute__((aligned(16))) unsigned char stage[kStreamers][16 * kMfmaRowBytes];
-    __shared__ f32x4_t red[kStreamers][64];
+// Variant for row lengths of 2048 or 4096: the weights are requested row by row (a load instruction fetches 1 KB of
+// one row, as the row-streaming kernels do; the operand layout above makes an instruction fetch 64 bytes from each
+// of 16 rows) and take the operand layout on their way through LDS: a wave writes 16 rows x 256 halfs at a time
+// (rows padded by 16 bytes, so that the sixteen rows a read touches fall into different banks) and reads the
+// 16 x 32 blocks back.
+constexpr int kMfmaRowBytes = kChunk + 16;
+// One workgroup per compute unit walks over its share of the 16-row blocks; wave w owns the
+// 512 halfs [512 w, 512 w + 512) of every row (NW = K / 512 waves).  The weights of the next block are requested
+// before the current one is multiplied, so the weight stream does not stop for the multiply / reduce phase of a
+// block.
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
+    __shared__ __attribute__((aligned(16))) unsigned char stage[NW][16 * kMfmaRowBytes];
+    __shared__ f32x4_t red[NW][64];
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
-    const int r0 = blockIdx.x * 16;
-    const size_t k0 = (size_t)wave * (CH * kChunk);
-    u32x4 w[CH][16];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-#pragma unroll
-        for (int j = 0; j < 16; ++j) w[c][j] = ld_stream16(a.W + (size_t)(r0 + j) * a.K + k0 + c * kChunk + lane * 8);
-    }
-    // operand blocks: step s of chunk c = k values 32 s + 8 (lane / 16) .. + 8 of row lane % 16
-    u32x4 op[CH][16];
+    const int nblocks = a.R / 16;
+    const int b0 = (int)(((long long)blockIdx.x * nblocks) / gridDim.x), b1 = (int)(((long long)(blockIdx.x + 1) * nblocks) / gridDim.x);
+    if (b0 >= b1) return;
+    const size_t k0 = (size_t)wave * kChunk;
     unsigned char* mine = stage[wave];
+    auto request = [&](u32x4 (&w)[16], int blk) {
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
+        for (int j = 0; j < 16; ++j) w[j] = ld_stream16(a.W + (size_t)(blk * 16 + j) * a.K + k0 + lane * 8);
+    };
+    auto load_x = [&](u32x4 (&x)[16], int t0) {
+        const int tok = t0 + (lane & 15) < a.batch ? t0 + (lane & 15) : a.batch - 1;
+        const half_t* xp = a.x + (size_t)tok * a.K + k0 + 8 * (lane >> 4);
+#pragma unroll
+        for (int s = 0; s < 16; ++s) x[s] = ld16(xp + 32 * s);
+    };
+    u32x4 wa[16], wb[16];
+    request(wa, b0);
+    // one block: rows -> operand layout through LDS (two halves of 256 halfs), multiply with every group of 16
+    // sequences, add the NW partial sums up
+    auto block = [&](u32x4 (&w)[16], int blk) {
+        u32x4 op[16];
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
             if ((lane >> 5) == hf) {
 #pragma unroll
-                for (int j = 0; j < 16; ++j) *reinterpret_cast<u32x4*>(mine + j * kMfmaRowBytes + (lane & 31) * 16) = w[c][j];
+                for (int j = 0; j < 16; ++j) *reinterpret_cast<u32x4*>(mine + j * kMfmaRowBytes + (lane & 31) * 16) = w[j];
             }
 #pragma unroll
             for (int s = 0; s < 8; ++s)
-                op[c][hf * 8 + s] = *reinterpret_cast<const u32x4*>(mine + (lane & 15) * kMfmaRowBytes + s * 64 + (lane >> 4) * 16);
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // the reads are done before the rows are overwritten
+                op[hf * 8 + s] = *reinterpret_cast<const u32x4*>(mine + (lane & 15) * kMfmaRowBytes + s * 64 + (lane >> 4) * 16);
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         }
-    }
-    for (int t0 = 0; t0 < a.batch; t0 += 16) {
-        const int tok = t0 + (lane & 15) < a.batch ? t0 + (lane & 15) : a.batch - 1;
-        const half_t* xp = a.x + (size_t)tok * a.K + k0 + 8 * (lane >> 4);
-        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
+        for (int t0 = 0; t0 < a.batch; t0 += 16) {
+            f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
             u32x4 x[16];
-#pragma unroll
-            for (int s = 0; s < 16; ++s) x[s] = ld16(xp + c * kChunk + 32 * s);
+            load_x(x, t0);         // cache hits
 #pragma unroll
             for (int s = 0; s < 16; ++s)
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, op[c][s]), __builtin_bit_cast(half8_t, x[s]), acc, 0, 0, 0);
-        }
-        __syncthreads();
-        red[wave][lane] = acc;
-        __syncthreads();
-        {
-            float sum = 0.f;
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, op[s]), __builtin_bit_cast(half8_t, x[s]), acc, 0, 0, 0);
+            __syncthreads();
+            red[wave][lane] = acc;
+            __syncthreads();
+            if (wave < 4) {
+                float sum = 0.f;
 #pragma unroll
-            for (int u = 0; u < kStreamers; ++u) sum += red[u][lane][wave];
-            const int seq = t0 + (lane & 15), row = r0 + 4 * (lane >> 4) + wave;
-            if (seq < a.batch) {
-                const size_t o = (size_t)seq * a.R + row;
-                if (a.out_f32 != nullptr) a.out_f32[o] = sum;
-                else a.out_f16[o] = (half_t)sum;
+                for (int u = 0; u < NW; ++u) sum += red[u][lane][wave];
+                const int seq = t0 + (lane & 15), row = blk * 16 + 4 * (lane >> 4) + wave;
+                if (seq < a.batch) {
+                    const size_t o = (size_t)seq * a.R + row;
+                    if (a.out_f32 != nullptr) a.out_f32[o] = sum;
+                    else a.out_f16[o] = (half_t)sum;
+                }
             }
         }
+    };
+    int blk = b0;
+    for (; blk + 1 < b1; blk += 2) {
+        request(wb, blk + 1);
+        block(wa, blk);
+        if (blk + 2 < b1) request(wa, blk + 2);
+        block(wb, blk + 1);
     }
+    if (blk < b1) block(wa, blk);
 }
 
 // (Fused add +) RMSNorm of the input rows, one wave per sequence: y = fp16(r * rstd * w), r = fp16(x + x_add) -> sum_out
@@ -1313,9 +1326,11 @@ int launch_batch_gemv_t(const BatchGemv& a, int grid, hipStream_t st) {
 }
 int launch_batch_mfma(const BatchMfma& a, hipStream_t st) {
     const int grid = a.R / 16;
-    if (env_int("CFPP_BATCH_MFMA_LDS", 1)) {
-        if (a.K == 4096) { hipLaunchKernelGGL((k_batch_mfma_lds<2>), dim3(grid), dim3(256), 0, st, a); return (int)hipGetLastError(); }
-        if (a.K == 2048) { hipLaunchKernelGGL((k_batch_mfma_lds<1>), dim3(grid), dim3(256), 0, st, a); return (int)hipGetLastError(); }
+    if (env_int("CFPP_BATCH_MFMA_PIPE", 1) && (a.K == 4096 || a.K == 2048)) {
+        const int wgs = streaming_grid() < grid ? streaming_grid() : grid;
+        if (a.K == 4096) hipLaunchKernelGGL((k_batch_mfma_pipe<8>), dim3(wgs), dim3(512), 0, st, a);
+        else hipLaunchKernelGGL((k_batch_mfma_pipe<4>), dim3(wgs), dim3(256), 0, st, a);
+        return (int)hipGetLastError();
     }
     switch (a.K / 256) {
         case 4: hipLaunchKernelGGL((k_batch_mfma<4>), dim3(grid), dim3(512), 0, st, a); break;
