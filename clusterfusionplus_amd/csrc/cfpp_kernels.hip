@@ -748,7 +748,7 @@ constexpr int kMfmaRowBytes = kChunk + 16;
 // 512 halfs [512 w, 512 w + 512) of every row (NW = K / 512 waves).  The weights of the next block are requested
 // before the current one is multiplied, so the weight stream does not stop for the multiply / reduce phase of a
 // block.
-template <int NW>
+template <int NW, bool ONE>
 __global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
     __shared__ __attribute__((aligned(16))) unsigned char stage[NW][16 * kMfmaRowBytes];
     __shared__ f32x4_t red[NW][64];
@@ -768,12 +768,8 @@ __global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
 #pragma unroll
         for (int s = 0; s < 16; ++s) x[s] = ld16(xp + 32 * s);
     };
-    u32x4 wa[16], wb[16];
-    request(wa, b0);
-    // one block: rows -> operand layout through LDS (two halves of 256 halfs), multiply with every group of 16
-    // sequences, add the NW partial sums up
-    auto block = [&](u32x4 (&w)[16], int blk) {
-        u32x4 op[16];
+    // rows -> operand layout through LDS (two halves of 256 halfs)
+    auto rearrange = [&](const u32x4 (&w)[16], u32x4 (&op)[16]) {
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
             if ((lane >> 5) == hf) {
@@ -785,37 +781,61 @@ __global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
                 op[hf * 8 + s] = *reinterpret_cast<const u32x4*>(mine + (lane & 15) * kMfmaRowBytes + s * 64 + (lane >> 4) * 16);
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         }
-        for (int t0 = 0; t0 < a.batch; t0 += 16) {
-            f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-            u32x4 x[16];
-            load_x(x, t0);         // cache hits
+    };
+    // multiply with one group of 16 sequences, add the NW partial sums up, store
+    auto multiply = [&](const u32x4 (&op)[16], const u32x4 (&x)[16], int blk, int t0) {
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s = 0; s < 16; ++s)
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, op[s]), __builtin_bit_cast(half8_t, x[s]), acc, 0, 0, 0);
-            __syncthreads();
-            red[wave][lane] = acc;
-            __syncthreads();
-            if (wave < 4) {
-                float sum = 0.f;
+        for (int s = 0; s < 16; ++s)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, op[s]), __builtin_bit_cast(half8_t, x[s]), acc, 0, 0, 0);
+        __syncthreads();
+        red[wave][lane] = acc;
+        __syncthreads();
+        if (wave < 4) {
+            float sum = 0.f;
 #pragma unroll
-                for (int u = 0; u < NW; ++u) sum += red[u][lane][wave];
-                const int seq = t0 + (lane & 15), row = blk * 16 + 4 * (lane >> 4) + wave;
-                if (seq < a.batch) {
-                    const size_t o = (size_t)seq * a.R + row;
-                    if (a.out_f32 != nullptr) a.out_f32[o] = sum;
-                    else a.out_f16[o] = (half_t)sum;
-                }
+            for (int u = 0; u < NW; ++u) sum += red[u][lane][wave];
+            const int seq = t0 + (lane & 15), row = blk * 16 + 4 * (lane >> 4) + wave;
+            if (seq < a.batch) {
+                const size_t o = (size_t)seq * a.R + row;
+                if (a.out_f32 != nullptr) a.out_f32[o] = sum;
+                else a.out_f16[o] = (half_t)sum;
             }
         }
     };
-    int blk = b0;
-    for (; blk + 1 < b1; blk += 2) {
-        request(wb, blk + 1);
-        block(wa, blk);
-        if (blk + 2 < b1) request(wa, blk + 2);
-        block(wb, blk + 1);
+    if constexpr (ONE) {
+        // up to 16 sequences: their input rows are the same for every block and stay in registers, so the only loads
+        // inside the loop are the weights, requested again as soon as the previous block has left the registers
+        u32x4 w[16], x0[16];
+        request(w, b0);
+        load_x(x0, 0);
+        for (int blk = b0; blk < b1; ++blk) {
+            u32x4 op[16];
+            rearrange(w, op);
+            if (blk + 1 < b1) request(w, blk + 1);
+            multiply(op, x0, blk, 0);
+        }
+    } else {
+        u32x4 wa[16], wb[16];
+        request(wa, b0);
+        auto block = [&](u32x4 (&w)[16], int blk) {
+            u32x4 op[16];
+            rearrange(w, op);
+            for (int t0 = 0; t0 < a.batch; t0 += 16) {
+                u32x4 x[16];
+                load_x(x, t0);         // cache hits
+                multiply(op, x, blk, t0);
+            }
+        };
+        int blk = b0;
+        for (; blk + 1 < b1; blk += 2) {
+            request(wb, blk + 1);
+            block(wa, blk);
+            if (blk + 2 < b1) request(wa, blk + 2);
+            block(wb, blk + 1);
+        }
+        if (blk < b1) block(wa, blk);
     }
-    if (blk < b1) block(wa, blk);
 }
 
 // (Fused add +) RMSNorm of the input rows, one wave per sequence: y = fp16(r * rstd * w), r = fp16(x + x_add) -> sum_out
@@ -1328,8 +1348,14 @@ int launch_batch_mfma(const BatchMfma& a, hipStream_t st) {
     const int grid = a.R / 16;
     if (env_int("CFPP_BATCH_MFMA_PIPE", 1) && (a.K == 4096 || a.K == 2048)) {
         const int wgs = streaming_grid() < grid ? streaming_grid() : grid;
-        if (a.K == 4096) hipLaunchKernelGGL((k_batch_mfma_pipe<8>), dim3(wgs), dim3(512), 0, st, a);
-        else hipLaunchKernelGGL((k_batch_mfma_pipe<4>), dim3(wgs), dim3(256), 0, st, a);
+        const bool one = a.batch <= 16 && env_int("CFPP_BATCH_MFMA_ONE", 1);
+        if (a.K == 4096) {
+            if (one) hipLaunchKernelGGL((k_batch_mfma_pipe<8, true>), dim3(wgs), dim3(512), 0, st, a);
+            else hipLaunchKernelGGL((k_batch_mfma_pipe<8, false>), dim3(wgs), dim3(512), 0, st, a);
+        } else {
+            if (one) hipLaunchKernelGGL((k_batch_mfma_pipe<4, true>), dim3(wgs), dim3(256), 0, st, a);
+            else hipLaunchKernelGGL((k_batch_mfma_pipe<4, false>), dim3(wgs), dim3(256), 0, st, a);
+        }
         return (int)hipGetLastError();
     }
     switch (a.K / 256) {
