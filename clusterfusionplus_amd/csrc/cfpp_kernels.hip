@@ -217,14 +217,18 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
 //                   (first weight tile in flight, then wait for kBarUp + g): the first down phase only needs
 //                   the first up phase of every workgroup, so a workgroup that is late with its MLP-up rows
 //                   holds up nobody until the second half of the down pass.
-//   attention wave: owns one (head, split) item: requests its first K/V tiles and RoPE coefficients, waits for
+//   attention wave: shares the QKV rows with the streaming waves when every wave still gets three tiles; owns at
+//                   most one (head, split) item (the host caps the KV splits so that one attention wave per
+//                   workgroup stays without: that one carries the MLP-up arrivals of its workgroup to the
+//                   device-wide counters): requests its first K/V tiles and RoPE coefficients, waits for
 //                   kBarQkv, runs the item at raised wave priority (the last wave of a head merges its
 //                   splits and bumps kBarHeads), then does the O-projection rows of stage C (all rows
 //                   requested, then wait for kBarHeads).  Attention is a chain of dependent memory round
 //                   trips; it and the O projection run beside the MLP-up / MLP-down streaming instead of in
 //                   front of it.
 //   all waves:      row reduction in LDS, bias, residual.
-// Nothing is reset at the end: counters zero themselves and flags carry a launch generation.  All workgroups must be
+// Nothing is reset at the end: counters zero themselves and flags carry a launch tag (from the generation word of the
+// workspace, or from the caller's step counter in the whole-model decoder).  All workgroups must be
 // co-resident (the host launches one per compute unit); every wait is bounded.
 struct FusedShared { int arrived[1 + kUpPhases]; };
 
