@@ -167,10 +167,10 @@ def bench_llama_layer(args, emit=True):
         "metric": "layer_latency_us", "value": round(us, 2), "unit": "us/layer", "n_gpus": 1, "steps": reps * nset, "warmup": args.warmup,
         "ms_per_step": round(us * 1e-3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": f"llama2_7b decoder layer (attention block + SwiGLU MLP block, 3 launches), batch-1 decode, context {S}, "
+        "config": {"workload": f"llama2_7b decoder layer (attention block + SwiGLU MLP block, 2 launches), batch-1 decode, context {S}, "
                                "graph replay over 8 weight sets", "context": S, "hidden": H, "ffn": F},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": None, "kernel": "k_fused (attention block) + k_gated_up + k_stage_c", "bytes_per_launch": nbytes,
+                     "traffic": None, "kernel": "k_fused (attention block) + k_gated_mlp", "bytes_per_launch": nbytes,
                      "launch_us": round(us, 2)},
         "cpu_baseline": None}
     if emit:

@@ -187,6 +187,63 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_up(LayerParams p) {
         });
 }
 
+// The whole gated MLP block in one launch: norm -> gate/up pairs in kUpPhases phases (a wave owns a contiguous range
+// of pairs of every phase; event kBarUp + g after phase g) -> down rows of stage C, which start on phase g of the
+// intermediate as soon as its event is complete, with their first weight tiles requested before the wait.  One
+// workgroup per compute unit, all co-resident; launch tag from the generation word, published again at the end.
+template <int NCH, int CPD, bool EX>
+__global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
+    __shared__ float park_mem[kStreamers][kParkRows];
+    __shared__ LnShared<NCH> lns;
+    __shared__ StageCShared shc;
+    __shared__ int arrived[kUpPhases];
+    const int gen = counter_peek(p.bar + kBarGen);
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int G = gridDim.x, b = blockIdx.x;
+    const int gw = b * kStreamers + wave, nw = G * kStreamers;
+    int* status = p.bar + kBarStatus;
+    if (threadIdx.x < kUpPhases) arrived[threadIdx.x] = 0;
+    RowPark park{park_mem[wave], 0};
+    const int F = p.F;
+    auto share = [&](int g, int& first, int& count) {      // this wave's pairs of phase g
+        const int lo = g == 0 ? 0 : up_phase_rows(CPD, g - 1, F), hi = up_phase_rows(CPD, g, F);
+        const int f0 = lo + (int)(((long long)gw * (hi - lo)) / nw), f1 = lo + (int)(((long long)(gw + 1) * (hi - lo)) / nw);
+        first = f0; count = f1 - f0;
+    };
+    int first, count;
+    share(0, first, count);
+    LnOwn<NCH, kStreamers> own;
+    ln_coop_load<NCH, kStreamers, false>(own, norm_spec(p), wave, lane);
+    __builtin_amdgcn_sched_barrier(0);   // the norm inputs go out first
+    RowTile<NCH, 2> t0;
+    if (count > 0) load_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, lane);
+    ln_coop_finish<NCH, kStreamers, false>(own, norm_spec(p), lns, wave, lane);
+    const int tag = first_lane(gen) + 1;
+    half2_t xr[NCH][4];
+    ln_fetch<NCH>(lns, 0, lane, xr);
+#pragma unroll
+    for (int g = 0; g < kUpPhases; ++g) {
+        const int f = first;
+        gemv_tiles<NCH, 2, EX>(
+            p.w_up, p.H, 2 * F, F, count, [=](int t) { return f + t; }, xr, lane, t0, park,
+            [&](const RowPark& pk, int k0) {
+                if (2 * lane + 1 < pk.n) st_agent(p.inter + f + k0 / 2 + lane, (half_t)(silu(pk.slot[2 * lane]) * pk.slot[2 * lane + 1]));
+            });
+        if (g + 1 < kUpPhases) {
+            share(g + 1, first, count);
+            if (count > 0) load_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, lane);     // in flight across the event
+        }
+        event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &arrived[g], kStreamers, tag);
+    }
+    const StageC c = make_stage_c(p);
+    stage_c_rows<NCH, CPD>(c, b, G, shc, true, wave, wave, kStreamers, lane,
+                           [&](int g) { event_wait(p.mbox, kBarUp + g, tag, status); }, [] {});
+    if (wave == 0) {
+        const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1, tag);
+        if (last && lane == 0) __hip_atomic_store(p.bar + kBarGen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 // one (head, split) item per wave
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_b(LayerParams p) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
@@ -1197,6 +1254,19 @@ int launch_gated_up(const Plan& pl, const LayerParams& p, int grid, hipStream_t 
     return CFPP_ERR_DIMS;
 }
 
+template <int NCH, int CPD>
+int launch_gated_mlp_t(const LayerParams& p, int grid, hipStream_t st) {
+    if (p.H == NCH * kChunk) hipLaunchKernelGGL((k_gated_mlp<NCH, CPD, true>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
+    else hipLaunchKernelGGL((k_gated_mlp<NCH, CPD, false>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
+    return launch_check();
+}
+int launch_gated_mlp(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
+#define X(a, b) if (pl.nch == a && pl.cpd == b) return launch_gated_mlp_t<a, b>(p, grid, st);
+    CFPP_SHAPE_CASES(X)
+#undef X
+    return CFPP_ERR_DIMS;
+}
+
 bool shape_supported(const Plan& pl) {
 #define X(a, b) if (pl.nch == a && pl.cpd == b) return true;
     CFPP_SHAPE_CASES(X)
@@ -1583,7 +1653,9 @@ int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t
 
 size_t cfpp_llama_mlp_workspace_bytes(int32_t hidden, int32_t ffn) {
     if (hidden <= 0 || ffn <= 0 || hidden % 8 || ffn % 8 || hidden > 8 * kChunk) return 0;
-    return align_up((size_t)ffn * 2, 256);
+    // intermediate row, then the words of the one-launch variant: flags / counters, group counters, mailboxes
+    return align_up((size_t)ffn * 2, 256) + 256 + align_up((size_t)(kBarExit + 1) * kEventGroups * kMailboxInts * 4, 256) +
+           (size_t)kMaxGrid * kMailboxInts * 4;
 }
 int cfpp_llama_mlp(const cfpp_llama_mlp_args* m, void* workspace, size_t workspace_bytes, void* stream) {
     if (!m || !workspace) return CFPP_ERR_NULL;
@@ -1608,6 +1680,14 @@ int cfpp_llama_mlp(const cfpp_llama_mlp_args* m, void* workspace, size_t workspa
     p.out = reinterpret_cast<half_t*>(m->output);
     p.c_base0 = p.x; p.c_use_o = 0; p.c_use_down = 1;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (env_int("CFPP_LLAMA_MLP_FUSED", 1)) {
+        // one launch: the down rows wait for the phases of the intermediate inside the kernel
+        char* ws = reinterpret_cast<char*>(workspace) + align_up((size_t)m->ffn * 2, 256);
+        p.bar = reinterpret_cast<int*>(ws);
+        p.grp = reinterpret_cast<int*>(ws + 256);
+        p.mbox = reinterpret_cast<int*>(ws + 256 + align_up((size_t)(kBarExit + 1) * kEventGroups * kMailboxInts * 4, 256));
+        return launch_gated_mlp(pl, p, fused_grid(), st);
+    }
     const int grid = streaming_grid();
     int rc = launch_gated_up(pl, p, grid, st);
     if (rc) return rc;

@@ -592,8 +592,21 @@ Tensor llama_mlp(Tensor input, Tensor rms_weight, Tensor gate_up_weight, Tensor 
     const size_t bytes = cfpp_llama_mlp_workspace_bytes(m.hidden, m.ffn);
     TORCH_CHECK(bytes > 0, "unsupported MLP dimensions (hidden ", H, ", ffn ", F, ")");
     hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
-    // the scratch (one fp16 row of F) comes from torch's caching allocator, which is stream ordered
-    Tensor ws = torch::empty({(int64_t)bytes + 256}, input.options().dtype(torch::kUInt8));
+    // zero-initialised scratch per (device, stream, geometry): its counters return to zero after every call
+    static std::mutex mu;
+    static std::map<std::tuple<int, void*, int, int>, Tensor> cache;
+    Tensor ws;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto key = std::make_tuple((int)input.device().index(), (void*)st, (int)H, (int)F);
+        auto it = cache.find(key);
+        if (it == cache.end()) {
+            ws = torch::zeros({(int64_t)bytes + 256}, input.options().dtype(torch::kUInt8));
+            cache[key] = ws;
+        } else {
+            ws = it->second;
+        }
+    }
     check_rc(cfpp_llama_mlp(&m, ws_ptr(ws), bytes, st), "llama_mlp");
     return out;
 }

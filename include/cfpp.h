@@ -149,10 +149,10 @@ int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t
 
 /* ---- LLaMA MLP block ---------------------------------------------------------------------------------
  * output = input + W_down (silu(Wg n) * (Wu n)),  n = RMSNorm(input; eps) * rms_w,  w_gate_up = [Wg; Wu] ([2F, H]),
- * w_down [H, F].  Two launches (norm + gated up rows, down rows + residual).  The reference fuses only the
+ * w_down [H, F].  One launch (norm, gated up rows in two phases, down rows + residual behind device-wide events).  The reference fuses only the
  * attention block of a LLaMA layer (its test leaves the MLP commented out, reference tests/test_llama.py:108-110);
  * this completes the layer its benchmark configuration describes.
- * Workspace: cfpp_llama_mlp_workspace_bytes, 256-byte aligned, no initialisation needed, one per stream. */
+ * Workspace: cfpp_llama_mlp_workspace_bytes, 256-byte aligned, zero-initialised once, one per stream. */
 typedef struct cfpp_llama_mlp_args {
     int32_t hidden, ffn;
     float eps;
