@@ -1012,8 +1012,11 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gemv_t(GemvT a) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) red[wave][lane * 8 + j] = acc[j];
     __syncthreads();
+    // thread t owns columns 2t and 2t + 1 of the panel from here on (kChunk == 2 * workgroup size)
+    static_assert(kChunk == 2 * kStreamers * 64, "two columns per thread");
+    const int c = 2 * threadIdx.x;
     float* mine = a.part + ((size_t)panel * a.slices + slice) * kChunk;
-    for (int c = threadIdx.x; c < kChunk; c += kStreamers * 64) st_agent(mine + c, red[0][c] + red[1][c] + red[2][c] + red[3][c]);
+    st_agent2(mine + c, red[0][c] + red[1][c] + red[2][c] + red[3][c], red[0][c + 1] + red[1][c + 1] + red[2][c + 1] + red[3][c + 1]);
     drain_memory_ops();
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -1024,14 +1027,25 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gemv_t(GemvT a) {
     __syncthreads();
     if (!last_flag) return;
     const int pc0 = (panel - sec * ppm) * kChunk;
-    for (int c = threadIdx.x; c < kChunk; c += kStreamers * 64) {
-        if (pc0 + c >= a.O) continue;
-        float sum = 0.f;
-        for (int sl = 0; sl < a.slices; ++sl) sum += ld_agent(a.part + ((size_t)panel * a.slices + sl) * kChunk + c);
-        const size_t o = (size_t)sec * a.O + pc0 + c;
-        if (a.out_f32 != nullptr) a.out_f32[o] = sum;
-        else a.out_f16[o] = (half_t)sum;
+    if (pc0 + c >= a.O) return;                       // O is a multiple of 8: both columns or none
+    // the slices in order, eight requests in flight at a time (requests past the last slice repeat it: a batch
+    // without branches, so that none of its loads waits for another)
+    const float* col0 = a.part + (size_t)panel * a.slices * kChunk + c;
+    float s0 = 0.f, s1 = 0.f;
+    for (int sl = 0; sl < a.slices; sl += 8) {
+        float u[8], v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int q = sl + i < a.slices ? sl + i : a.slices - 1;
+            ld_agent2(col0 + (size_t)q * kChunk, u[i], v[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (sl + i < a.slices) { s0 += u[i]; s1 += v[i]; }
     }
+    const size_t o = (size_t)sec * a.O + pc0 + c;
+    if (a.out_f32 != nullptr) { a.out_f32[o] = s0; a.out_f32[o + 1] = s1; }
+    else { a.out_f16[o] = (half_t)s0; a.out_f16[o + 1] = (half_t)s1; }
 }
 
 // stage B with GPT-J pairing of the rotary dims
