@@ -966,6 +966,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_norm(BatchNorm a) {
 struct GemvT {
     const half_t* W; int K, O, nsec;
     const half_t* x;                 // [K] fp16
+    const half_t* norm_w; float eps; // not null: x stands for fp16(x * rstd(x) * norm_w), the RMSNorm of the row
     float* part;                     // [panels][slices][512]
     int* cnt;                        // [panels], zero between launches
     float* out_f32; half_t* out_f16; // [nsec O], one of the two
@@ -988,10 +989,22 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gemv_t(GemvT a) {
     float acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    float rstd = 1.f;
+    if (a.norm_w != nullptr) {         // every wave takes the statistics of the whole row itself: 2 bytes per k
+        float ss = 0.f;
+        for (int c0 = lane * 8; c0 < a.K; c0 += kChunk) {
+            float f[8];
+            unpack8(ld16(a.x + c0), f);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ss += f[j] * f[j];
+        }
+        rstd = 1.0f / sqrtf(wave_sum(ss) / (float)a.K + a.eps);
+    }
     constexpr int kRows = 8;           // rows requested together
     for (int kb = k0; kb < k1; kb += 64) {
         const int n = k1 - kb < 64 ? k1 - kb : 64;
-        const float xv = lane < n ? (float)a.x[kb + lane] : 0.f;     // x[kb + lane]; rows past the range get 0
+        float xv = lane < n ? (float)a.x[kb + lane] : 0.f;           // x[kb + lane]; rows past the range get 0
+        if (a.norm_w != nullptr && lane < n) xv = (float)(half_t)(xv * rstd * (float)a.norm_w[kb + lane]);
         for (int r = 0; r < n; r += kRows) {
             u32x4 w[kRows];
 #pragma unroll
@@ -1592,7 +1605,7 @@ int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_
 }
 
 // The reference's plain llama_decoder_layer op: as cfpp_llama_attention_decode without a residual, with weights stored
-// [in, out] and GPT-J pairing of the rotary dims.  Four launches: norm, QKV products, attention items, O products.
+// [in, out] and GPT-J pairing of the rotary dims.  Three launches: QKV products (with the norm of the input row), attention items, O products.
 size_t cfpp_llama_plain_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim) {
     const size_t base = cfpp_llama_workspace_bytes(hidden, heads, head_dim);
     if (base == 0) return 0;
@@ -1630,10 +1643,13 @@ int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t
     half_t* xn = reinterpret_cast<half_t*>(reinterpret_cast<char*>(cnt) + align_up((size_t)3 * ppm * 4, 256));
     auto h = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
 
-    BatchNorm n{};
-    n.x = h(a->input); n.x_add = nullptr; n.norm_w = h(a->rms_w); n.sum_out = nullptr; n.y = xn;
-    n.eps = a->eps; n.K = H; n.batch = 1;
-    if ((rc = launch_batch_norm(pl.nch, n, st))) return rc;
+    const bool norm_inside = env_int("CFPP_PLAIN_NORM_INSIDE", 1) != 0;
+    if (!norm_inside) {
+        BatchNorm n{};
+        n.x = h(a->input); n.x_add = nullptr; n.norm_w = h(a->rms_w); n.sum_out = nullptr; n.y = xn;
+        n.eps = a->eps; n.K = H; n.batch = 1;
+        if ((rc = launch_batch_norm(pl.nch, n, st))) return rc;
+    }
 
     cfpp_neox_weights w{};
     w.ln_w = a->rms_w; w.ln_b = a->rms_w; w.w_qkv = a->w_qkv; w.b_qkv = a->rms_w; w.w_o = a->w_o; w.b_o = a->rms_w;
@@ -1649,20 +1665,22 @@ int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t
     p.qkv_head_stride = d.head_dim; p.qkv_k_off = H; p.qkv_v_off = 2 * H;
     p.append_kv = 0;
 
-    auto gemv = [&](const half_t* W, int nsec, const half_t* x, float* out_f32, half_t* out_f16) {
+    auto gemv = [&](const half_t* W, int nsec, const half_t* x, const half_t* norm_w, float* out_f32, half_t* out_f16) {
         GemvT g{};
-        g.W = W; g.K = H; g.O = H; g.nsec = nsec; g.x = x; g.part = part; g.cnt = cnt;
+        g.W = W; g.K = H; g.O = H; g.nsec = nsec; g.x = x; g.norm_w = norm_w; g.eps = a->eps; g.part = part; g.cnt = cnt;
         g.out_f32 = out_f32; g.out_f16 = out_f16;
         const int panels = nsec * ppm;
         g.slices = grid / panels < 1 ? 1 : (grid / panels > 64 ? 64 : grid / panels);
         hipLaunchKernelGGL(k_gemv_t, dim3(panels * g.slices), dim3(kStreamers * 64), 0, st, g);
         return (int)hipGetLastError();
     };
-    if ((rc = gemv(h(a->w_qkv), 3, xn, p.qkv_raw, nullptr))) return rc;
+    // the QKV launch normalises the input row on its way in
+    if ((rc = norm_inside ? gemv(h(a->w_qkv), 3, h(a->input), h(a->rms_w), p.qkv_raw, nullptr)
+                          : gemv(h(a->w_qkv), 3, xn, nullptr, p.qkv_raw, nullptr))) return rc;
     const int bgrid = (p.heads * split_bound(a->seq_len, p.max_split) + kStreamers - 1) / kStreamers;
     hipLaunchKernelGGL(k_stage_b_pairs, dim3(bgrid), dim3(kStreamers * 64), 0, st, p);
     if ((rc = (int)hipGetLastError())) return rc;
-    return gemv(h(a->w_o), 1, p.attn_vec, nullptr, reinterpret_cast<half_t*>(a->output));
+    return gemv(h(a->w_o), 1, p.attn_vec, nullptr, nullptr, reinterpret_cast<half_t*>(a->output));
 }
 
 size_t cfpp_llama_mlp_workspace_bytes(int32_t hidden, int32_t ffn) {
