@@ -805,13 +805,14 @@ __global__ __launch_bounds__(512) void k_batch_mfma(BatchMfma a) {
 // (rows padded by 16 bytes, so that the sixteen rows a read touches fall into different banks) and reads the
 // 16 x 32 blocks back.
 constexpr int kMfmaRowBytes = kChunk + 16;
+constexpr int kMfmaFullRowBytes = 2 * kChunk + 16;     // a wave's whole 512-half share of a row, same padding
 // One workgroup per compute unit walks over its share of the 16-row blocks; wave w owns the
 // 512 halfs [512 w, 512 w + 512) of every row (NW = K / 512 waves).  The weights of the next block are requested
 // before the current one is multiplied, so the weight stream does not stop for the multiply / reduce phase of a
 // block.
 template <int NW, bool ONE>
 __global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
-    __shared__ __attribute__((aligned(16))) unsigned char stage[NW][16 * kMfmaRowBytes];
+    __shared__ __attribute__((aligned(16))) unsigned char stage[NW][16 * (ONE ? kMfmaFullRowBytes : kMfmaRowBytes)];
     __shared__ f32x4_t red[NW][64];
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
     const int nblocks = a.R / 16;
@@ -866,14 +867,29 @@ __global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
     };
     if constexpr (ONE) {
         // up to 16 sequences: their input rows are the same for every block and stay in registers, so the only loads
-        // inside the loop are the weights, requested again as soon as the previous block has left the registers
+        // inside the loop are the weights.  A wave stages its whole 512-half share of the 16 rows at once, and a row's
+        // registers take the next block's row as soon as the row is in LDS: the number of requests in flight stays at
+        // fifteen or sixteen instead of draining to none once per block
         u32x4 w[16], x0[16];
         request(w, b0);
         load_x(x0, 0);
         for (int blk = b0; blk < b1; ++blk) {
             u32x4 op[16];
-            rearrange(w, op);
-            if (blk + 1 < b1) request(w, blk + 1);
+            const bool more = blk + 1 < b1;
+            {
+                const half_t* next = a.W + (size_t)((more ? blk + 1 : blk) * 16) * a.K + k0 + lane * 8;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    *reinterpret_cast<u32x4*>(mine + j * kMfmaFullRowBytes + lane * 16) = w[j];
+                    if (more) w[j] = ld_stream16(next + (size_t)j * a.K);
+                    asm volatile("" ::: "memory");        // keep the store / request pairs in this order
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+                for (int s = 0; s < 16; ++s)
+                    op[s] = *reinterpret_cast<const u32x4*>(mine + (lane & 15) * kMfmaFullRowBytes + s * 64 + (lane >> 4) * 16);
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            }
             multiply(op, x0, blk, 0);
         }
     } else {
