@@ -65,16 +65,15 @@ struct LayerParams {
     int cache_rows;
     const float *cos, *sin;
     int rope_stride;
+    int rope_half_table;    // rotate-half RoPE: 0 = cos/sin hold one entry per rotary dim and dim d uses entry d (GPT-NeoX ops);
+                            // 1 = they hold rot/2 entries, the angles of the pairs, and dims d and d + rot/2 share entry d
     int seq_len;
     const int* d_seq_len;
     int max_split;      // cap on the KV splits per head (<= kMaxSplit)
-    int row_walk_strided;   // streaming waves take interleaved instead of contiguous row ranges
     const int* kv_rows;     // paged caches: cache row r of this sequence lives in row kv_rows[r] of k_cache / v_cache (null: r itself)
     const int* tag_src;     // launch tags from a counter the caller advances between launches (null: from kBarGen)
     int tag_mul, tag_add;   // tag = tag_src[0] * tag_mul + tag_add + 1
-    int qkv_all_waves;      // fused kernel: the attention waves share the QKV rows with the streaming waves
     int arrival_agents;     // an idle attention wave carries the streaming waves' MLP-up arrivals to the device-wide counters
-    int dyn_up;             // MLP-up tiles handed out dynamically within teams of workgroups: 1 yes, 0 no, -1 by size
     // layer family switches (defaults = GPT-NeoX): RMSNorm instead of LayerNorm; where head h's raw q, k, v sit in
     // qkv_raw (NeoX interleaves [h][q|k|v][D]: stride 3D, offsets D and 2D; LLaMA stacks [q;k;v]: stride D,
     // offsets H and 2H); whether split 0 appends the new K/V row to the caches
@@ -97,10 +96,16 @@ struct LayerParams {
     const half_t* c_base0;   // residual terms added to the output (nullable)
     const half_t* c_base1;
     int c_use_o, c_use_down;
-    long long* trace;   // debugging: per-workgroup phase timestamps of the fused kernel (null = off)
+    int* host_status;   // nullable: a word in pinned host memory that receives every failure flag as well, so that the
+                        // host sees a failed launch without reading device memory
+#ifdef CFPP_TRACE
+    long long* trace;   // per-workgroup phase timestamps of the fused kernel (null = off); profiling builds only
+#endif
 };
 
+// Phase timestamps of the fused kernel exist in profiling builds (-DCFPP_TRACE) only.
 constexpr int kTraceSlots = 16;
+#ifdef CFPP_TRACE
 __device__ __forceinline__ void trace_value(const LayerParams& p, int slot, long long v) {
     if (p.trace != nullptr && (threadIdx.x & 63) == 0)
         p.trace[((size_t)blockIdx.x * kMaxWaves + (threadIdx.x >> 6)) * kTraceSlots + slot] = v;
@@ -109,6 +114,10 @@ __device__ __forceinline__ void trace_mark(const LayerParams& p, int slot) {
     if (p.trace != nullptr && (threadIdx.x & 63) == 0)
         p.trace[((size_t)blockIdx.x * kMaxWaves + (threadIdx.x >> 6)) * kTraceSlots + slot] = wall_clock64();
 }
+#else
+__device__ __forceinline__ void trace_value(const LayerParams&, int, long long) {}
+__device__ __forceinline__ void trace_mark(const LayerParams&, int) {}
+#endif
 
 // ------------------------------------------------------------------------------------------------
 // loads / conversions
@@ -232,8 +241,12 @@ __device__ __forceinline__ void counter_add(int* ctr, int v) {
 __device__ __forceinline__ int counter_peek(const int* ctr) {
     return __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void raise_status(int* status, int flag) {
-    __hip_atomic_fetch_or(status, flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Failure flags go to the workspace's status word and, when the launch has one, to a word in pinned host memory
+// (a plain system-scope store of the flag: the host only asks whether it is non-zero).
+struct StatusSink { int* dev; int* host; };
+__device__ __forceinline__ void raise_status(const StatusSink& s, int flag) {
+    __hip_atomic_fetch_or(s.dev, flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (s.host != nullptr) __hip_atomic_store(s.host, flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 // Arrivals are counted hierarchically, because a thousand waves adding to one address serialise at the
 // memory side (tens of nanoseconds each) and every one of them waits for its return value: first in LDS
@@ -282,7 +295,7 @@ __device__ __forceinline__ bool event_arrive(int* bar, int* grp, int* mbox, int 
 // One lane polls this workgroup's mailbox line, the wave leaves together.  Data published before the
 // arrivals must be read with ld_agent / ld_agent16.  A wait that expires raises a status flag and
 // falls through.
-__device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, int* status) {
+__device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, const StatusSink& status) {
     if ((threadIdx.x & 63) == 0) {
         const int* f = mbox + blockIdx.x * kMailboxInts + slot;
         int spins = 0;
@@ -295,13 +308,23 @@ __device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, i
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
-__device__ __forceinline__ int load_seq_len(const LayerParams& p) {
+__device__ __forceinline__ StatusSink status_sink(const LayerParams& p) { return StatusSink{p.bar + kBarStatus, p.host_status}; }
+
+// The number of valid cache rows S of this step.  A host-side length may equal the cache rows (the append is then
+// skipped, k_new / v_new are still returned).  A device-side length, or RoPE tables indexed by the position
+// (rope_stride > 0, one table row per cache row), need S < cache_rows: the step reads table row S and appends cache
+// row S.  Anything else raises kStatusSeq; the step then runs on a clamped length without appending, so that no
+// access leaves the caches or the tables, and its results mean nothing.
+struct SeqLen { int S; bool ok; };
+__device__ __forceinline__ SeqLen load_seq_len(const LayerParams& p) {
     int S = p.d_seq_len ? *p.d_seq_len : p.seq_len;
-    if (S < 0 || S > p.cache_rows) {
-        if (threadIdx.x == 0 && blockIdx.x == 0) raise_status(p.bar + kBarStatus, kStatusSeq);
-        S = S < 0 ? 0 : p.cache_rows;
+    const int limit = (p.d_seq_len != nullptr || p.rope_stride > 0) ? p.cache_rows - 1 : p.cache_rows;
+    const bool ok = S >= 0 && S <= limit;
+    if (!ok) {
+        if (threadIdx.x == 0 && blockIdx.x == 0) raise_status(status_sink(p), kStatusSeq);
+        S = (S < 0 || limit < 0) ? 0 : limit;
     }
-    return S;
+    return SeqLen{S, ok};
 }
 // KV splits per head for a sequence length: about kSplitRows cache rows per item
 __device__ __forceinline__ int effective_split(const LayerParams& p, int S) {
@@ -693,10 +716,15 @@ struct StageARpi { static constexpr int value = (16 / NCH) > 0 ? (16 / NCH) : 1;
 // rope_load8 requests the lane's own values and their rotation partners together (one memory round trip).
 // PAIRS: dim d rotates with d +- rot/2 (false, NeoX) or with its neighbour d ^ 1 (true, GPT-J: even dims take
 // -sin, odd dims +sin, and the tables are indexed by the dim itself; reference include/5090/llama/kernel.cuh:280-313).
+// Rotate-half tables come in two shapes.  The Pythia ops read cos[d] / sin[d] for every d < rot (reference
+// include/5090/pythia_2b8/kernel.cuh:395-399): the two halves of the table need not repeat, and the reference's
+// own unit test draws an independent angle per entry (tests/test_pythia.py:24-42).  The sglang LLaMA ops hold only
+// the rot/2 angles of the pairs and read entry d mod rot/2 (reference include/5090/llama/kernel_sglang.cuh:292-293):
+// `half_table`.
 struct RopeCoeffs { float c[8], sg[8]; };
 template <bool PAIRS = false>
 __device__ __forceinline__ void rope_coeffs(int d0, int rot, const float* __restrict__ cs, const float* __restrict__ sn,
-                                            bool act, RopeCoeffs& rc) {
+                                            bool act, bool half_table, RopeCoeffs& rc) {
     const int hr = rot >> 1;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -706,7 +734,7 @@ __device__ __forceinline__ void rope_coeffs(int d0, int rot, const float* __rest
             rc.c[j] = rotd ? cs[d] : 1.f;
             rc.sg[j] = rotd ? ((d & 1) ? sn[d] : -sn[d]) : 0.f;
         } else {
-            const int t = d < hr ? d : d - hr;       // both halves use the angle of the pair (entries [0, rot/2) of the table)
+            const int t = (half_table && d >= hr) ? d - hr : d;
             rc.c[j] = rotd ? cs[t] : 1.f;
             rc.sg[j] = rotd ? (d < hr ? -sn[t] : sn[t]) : 0.f;
         }
@@ -758,6 +786,7 @@ constexpr int kAttnTileRows = 4 * kAttnT;
 struct KvTile { u32x4 k[kAttnT], v[kAttnT]; };
 struct AttnItem {
     int head, sp, nsplit, S, begin, end, ntiles;
+    bool append_ok;     // the sequence length was valid: split 0 may append the new row
     KvTile t0, t1;
     RopeCoeffs rc;
 };
@@ -779,8 +808,9 @@ __device__ __forceinline__ void attn_load_tile(const LayerParams& p, const AttnI
     }
 }
 template <bool PAGED = false, bool PAIRS = false>
-__device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it, int head, int sp, int nsplit, int S, int lane) {
-    it.head = head; it.sp = sp; it.nsplit = nsplit; it.S = S;
+__device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it, int head, int sp, int nsplit, SeqLen sl, int lane) {
+    const int S = sl.S;
+    it.head = head; it.sp = sp; it.nsplit = nsplit; it.S = S; it.append_ok = sl.ok;
     const int chunk = (S + nsplit - 1) / nsplit;
     it.begin = sp * chunk;
     it.end = (it.begin + chunk < S) ? it.begin + chunk : S;
@@ -791,7 +821,7 @@ __device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it
     const bool act = sub * 8 < p.D;
     const float* __restrict__ cs = p.cos + (size_t)S * p.rope_stride;   // stride 0: the row is the position
     const float* __restrict__ sn = p.sin + (size_t)S * p.rope_stride;
-    rope_coeffs<PAIRS>(act ? sub * 8 : 0, p.rot, cs, sn, act, it.rc);
+    rope_coeffs<PAIRS>(act ? sub * 8 : 0, p.rot, cs, sn, act, p.rope_half_table != 0, it.rc);
 }
 
 // nwg_to_signal > 0 (fused kernel): a completed head counts towards the kBarHeads event of that many workgroups.
@@ -826,12 +856,12 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
             *reinterpret_cast<u32x4*>(p.k_new + o) = kp;
             *reinterpret_cast<u32x4*>(p.v_new + o) = vp;
             if (PAGED) {
-                if (p.append_kv) {
+                if (p.append_kv && it.append_ok) {
                     const size_t slot = (size_t)p.kv_rows[S];
                     *reinterpret_cast<u32x4*>(p.k_cache + slot * H + o) = kp;
                     *reinterpret_cast<u32x4*>(p.v_cache + slot * H + o) = vp;
                 }
-            } else if (p.append_kv && S < p.cache_rows) {
+            } else if (p.append_kv && it.append_ok && S < p.cache_rows) {
                 *reinterpret_cast<u32x4*>(p.k_cache + (size_t)S * H + o) = kp;
                 *reinterpret_cast<u32x4*>(p.v_cache + (size_t)S * H + o) = vp;
             }

@@ -26,24 +26,18 @@ namespace {
 // between the two variants makes the compiler keep two copies of the in-flight tiles.
 
 // The rows a streaming wave takes from a row range [lo, hi) shared by `nw` waves, as tiles of RPI rows:
-// tile t covers rows first + t*step + j*sit, j < RPI, below `end`.
-//   blocked  (default): wave w owns the contiguous rows lo + [w n / nw, (w+1) n / nw) in units of RPI
-//            rows; it walks through memory sequentially, so it meets every memory channel and page in
-//            turn and channel conflicts average out within the wave.
-//   strided: wave w owns tiles w, w + nw, ...; every access of a wave is nw*RPI rows from the last one.
+// tile t covers rows first + t*step + j*sit, j < RPI, below `end`.  Wave w owns the contiguous rows
+// lo + [w n / nw, (w+1) n / nw) in units of RPI rows; it walks through memory sequentially, so it meets every
+// memory channel and page in turn and channel conflicts average out within the wave.  (Interleaved ownership,
+// wave w taking tiles w, w + nw, ..., was measured slower.)
 struct RowWalk { int first, step, sit, end, ntiles; };
 template <int RPI>
-__device__ __forceinline__ RowWalk row_walk(bool strided, int w, int nw, int lo, int hi) {
+__device__ __forceinline__ RowWalk row_walk(int w, int nw, int lo, int hi) {
     const int units = (hi - lo + RPI - 1) / RPI;
     RowWalk rw;
-    if (strided) {
-        rw.first = lo + w * RPI; rw.step = nw * RPI; rw.sit = 1; rw.end = hi;
-        rw.ntiles = w < units ? (units - w + nw - 1) / nw : 0;
-    } else {
-        const int u0 = (int)(((long long)w * units) / nw), u1 = (int)(((long long)(w + 1) * units) / nw);
-        rw.first = lo + u0 * RPI; rw.step = RPI; rw.sit = 1; rw.ntiles = u1 - u0;
-        rw.end = lo + u1 * RPI < hi ? lo + u1 * RPI : hi;
-    }
+    const int u0 = (int)(((long long)w * units) / nw), u1 = (int)(((long long)(w + 1) * units) / nw);
+    rw.first = lo + u0 * RPI; rw.step = RPI; rw.sit = 1; rw.ntiles = u1 - u0;
+    rw.end = lo + u1 * RPI < hi ? lo + u1 * RPI : hi;
     return rw;
 }
 template <int RPI>
@@ -140,8 +134,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_a(LayerParams p) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int gw = blockIdx.x * kStreamers + wave, nw = gridDim.x * kStreamers;
     RowPark park{park_mem[wave], 0};
-    const bool strided = p.row_walk_strided != 0;
-    const RowWalk qw = row_walk<StageARpi<NCH>::value>(strided, gw, nw, 0, 3 * p.H);
+    const RowWalk qw = row_walk<StageARpi<NCH>::value>(gw, nw, 0, 3 * p.H);
     LnOwn<NCH, kStreamers> own;
     ln_coop_load<NCH, kStreamers, true>(own, norm_spec(p), wave, lane);
     __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
@@ -151,7 +144,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_a(LayerParams p) {
     half2_t xr[NCH][4];
     ln_fetch<NCH>(lns, 0, lane, xr);
     qkv_rows<NCH, EX>(p, xr, qw, lane, t0, park);
-    const RowWalk uw = row_walk<kUpRpi>(strided, gw, nw, 0, p.F);
+    const RowWalk uw = row_walk<kUpRpi>(gw, nw, 0, p.F);
     RowTile<NCH, kUpRpi> u0;
     up_prefetch<NCH, EX>(p, uw, lane, u0);
     ln_fetch<NCH>(lns, 1, lane, xr);
@@ -201,7 +194,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
     const int G = gridDim.x, b = blockIdx.x;
     const int gw = b * kStreamers + wave, nw = G * kStreamers;
-    int* status = p.bar + kBarStatus;
+    const StatusSink status = status_sink(p);
     if (threadIdx.x < kUpPhases) arrived[threadIdx.x] = 0;
     RowPark park{park_mem[wave], 0};
     const int F = p.F;
@@ -247,12 +240,12 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
 // one (head, split) item per wave
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_b(LayerParams p) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
-    const int S = load_seq_len(p);
-    const int nsplit = effective_split(p, S);
+    const SeqLen sl = load_seq_len(p);
+    const int nsplit = effective_split(p, sl.S);
     const int item = blockIdx.x * kStreamers + wave;
     if (item < p.heads * nsplit) {
         AttnItem it;
-        attn_prefetch(p, it, item / nsplit, item % nsplit, nsplit, S, lane);
+        attn_prefetch(p, it, item / nsplit, item % nsplit, nsplit, sl, lane);
         attention_item(p, it, lane, 0, 0);
     }
 }
@@ -311,7 +304,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const int G = gridDim.x, b = blockIdx.x;
     const int nsw = G * kStreamers;                 // streaming waves in the grid
-    int* status = p.bar + kBarStatus;
+    const StatusSink status = status_sink(p);
     if (threadIdx.x <= kUpPhases) q.arrived[threadIdx.x] = 0;
     __syncthreads();
     trace_mark(p, 0);
@@ -327,9 +320,9 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
     // (only when that leaves every wave three tiles or more: with fewer, the attention waves start their items later
     // than the shorter QKV pass gains)
     const int qkv_units = (3 * p.H + RPIA - 1) / RPIA;
-    const bool qkv8 = p.qkv_all_waves > 0 || (p.qkv_all_waves < 0 && qkv_units >= 3 * G * kFusedWaves);
-    const RowWalk qw = qkv8 ? row_walk<RPIA>(false, b * kFusedWaves + wave, G * kFusedWaves, 0, 3 * p.H)
-                            : row_walk<RPIA>(false, b * kStreamers + (wave < kStreamers ? wave : 0), nsw, 0,
+    const bool qkv8 = qkv_units >= 3 * G * kFusedWaves;
+    const RowWalk qw = qkv8 ? row_walk<RPIA>(b * kFusedWaves + wave, G * kFusedWaves, 0, 3 * p.H)
+                            : row_walk<RPIA>(b * kStreamers + (wave < kStreamers ? wave : 0), nsw, 0,
                                              wave < kStreamers ? 3 * p.H : 0);
     const int qkv_arrivals = qkv8 ? kFusedWaves : kStreamers;
     const int hw = wave - kStreamers;
@@ -342,8 +335,8 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
         ln_coop_finish<NCH, kFusedWaves, true>(own, norm_spec(p), lns, wave, lane);
     }
     const int tag = first_lane(gen) + 1;
-    const int S = load_seq_len(p);
-    const int nsplit = effective_split(p, S);
+    const SeqLen sl = load_seq_len(p);
+    const int nsplit = effective_split(p, sl.S);
     const int nitems = p.heads * nsplit;
     const int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
     trace_mark(p, 1);
@@ -385,7 +378,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
         // (only when a wave can expect four tiles or more per phase: with fewer, the static shares are
         // already as fine as the tickets, and the ticket round trips cost more than they balance)
         TileTeam utm = make_team<kUpRpi>(p, 1, 0, up_phase_rows(CPD, 0, p.F), b, G, wave);
-        const bool dynamic = p.dyn_up > 0 || (p.dyn_up < 0 && utm.ntiles >= 4 * utm.nw);
+        const bool dynamic = utm.ntiles >= 4 * utm.nw;
         if (dynamic) {
             TeamTiles<NCH, kUpRpi> ut;
             team_prefetch<NCH, kUpRpi, EX>(p.w_up, p.H, utm, lane, ut);
@@ -404,7 +397,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
             }
         } else {
             RowTile<NCH, kUpRpi> u0;
-            RowWalk uw = row_walk<kUpRpi>(false, b * kStreamers + wave, nsw, 0, up_phase_rows(CPD, 0, p.F));
+            RowWalk uw = row_walk<kUpRpi>(b * kStreamers + wave, nsw, 0, up_phase_rows(CPD, 0, p.F));
             up_prefetch<NCH, EX>(p, uw, lane, u0);
             event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
             trace_mark(p, 2);
@@ -413,7 +406,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
             for (int g = 0; g < kUpPhases; ++g) {
                 up_rows<NCH, EX>(p, xr, uw, lane, u0, spark);
                 if (g + 1 < kUpPhases) {
-                    uw = row_walk<kUpRpi>(false, b * kStreamers + wave, nsw, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F));
+                    uw = row_walk<kUpRpi>(b * kStreamers + wave, nsw, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F));
                     up_prefetch<NCH, EX>(p, uw, lane, u0);
                 }
                 stream_arrive(kBarUp + g, &q.arrived[1 + g], agent_up);
@@ -433,7 +426,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
         }
         if (hw < attn_count) {
             AttnItem it;
-            attn_prefetch(p, it, (b + hw * G) / nsplit, (b + hw * G) % nsplit, nsplit, S, lane);
+            attn_prefetch(p, it, (b + hw * G) / nsplit, (b + hw * G) % nsplit, nsplit, sl, lane);
             event_wait(p.mbox, kBarQkv, tag, status);
             __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
             trace_mark(p, 3);
@@ -499,7 +492,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __res
     constexpr int RPIA = StageARpi<NCH>::value;
     __shared__ float park_mem[NWV][kParkRows];
     RowPark park{park_mem[wave], 0};
-    const RowWalk rw = row_walk<RPIA>(false, gw, nw, 0, vocab);   // contiguous rows per wave
+    const RowWalk rw = row_walk<RPIA>(gw, nw, 0, vocab);   // contiguous rows per wave
     __shared__ LnShared<NCH> lns;
     LnOwn<NCH, NWV> own;
     const NormSpec ns{x, nullptr, ln_w, ln_b, nullptr, nullptr, H, 0, eps};
@@ -611,7 +604,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_gemv(BatchGemv a) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
     const int gw = blockIdx.x * kStreamers + wave, nw = gridDim.x * kStreamers;
     constexpr int RPI = 2;
-    const RowWalk rw = row_walk<RPI>(false, gw, nw, 0, a.R);
+    const RowWalk rw = row_walk<RPI>(gw, nw, 0, a.R);
     const int nrows = rw.end > rw.first ? rw.end - rw.first : 0;
     for (int t0 = 0; t0 < a.batch; t0 += kBatchTile) {
         const int nb = a.batch - t0 < kBatchTile ? a.batch - t0 : kBatchTile;
@@ -1080,12 +1073,12 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gemv_t(GemvT a) {
 // stage B with GPT-J pairing of the rotary dims
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_b_pairs(LayerParams p) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
-    const int S = load_seq_len(p);
-    const int nsplit = effective_split(p, S);
+    const SeqLen sl = load_seq_len(p);
+    const int nsplit = effective_split(p, sl.S);
     const int item = blockIdx.x * kStreamers + wave;
     if (item < p.heads * nsplit) {
         AttnItem it;
-        attn_prefetch<false, true>(p, it, item / nsplit, item % nsplit, nsplit, S, lane);
+        attn_prefetch<false, true>(p, it, item / nsplit, item % nsplit, nsplit, sl, lane);
         attention_item<false, true>(p, it, lane, 0, 0);
     }
 }
@@ -1111,7 +1104,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_attn(LayerParams p, B
     const int start = b.indptr[seq];
     int S = b.indptr[seq + 1] - 1 - start;
     if (S < 0) {
-        if (lane == 0) raise_status(p.bar + kBarStatus, kStatusSeq);
+        if (lane == 0) raise_status(status_sink(p), kStatusSeq);
         return;
     }
     const int nsplit = effective_split(p, S);
@@ -1131,15 +1124,22 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_attn(LayerParams p, B
     q.part_acc += (size_t)seq * p.heads * kMaxSplit * p.D;
     q.head_cnt += (size_t)seq * p.heads;
     AttnItem it;
-    attn_prefetch<true>(q, it, head, sp, nsplit, S, lane);
+    attn_prefetch<true>(q, it, head, sp, nsplit, SeqLen{S, true}, lane);
     attention_item<true>(q, it, lane, 0, 0);
 }
 
 
+// What the library keeps per device, set up at the first call on that device.
 struct DeviceInfo {
     int cus = 0;
     bool ok = false;
+    int* host_status = nullptr;        // one word of pinned host memory: device-side failure flags land here as well
+    int* host_status_dev = nullptr;    // the device's address of that word
+    std::map<const void*, int> blocks_per_cu;   // occupancy of the one-launch kernels, by kernel
+    void* static_scratch = nullptr;    // address of this device's copy of the file-scope scratch array
+    unsigned long long static_key = 0; // geometry of the last call that used it (0: never used)
 };
+std::mutex g_device_mu;
 
 DeviceInfo& device_info() {
     static DeviceInfo info[64];
@@ -1147,23 +1147,45 @@ DeviceInfo& device_info() {
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     DeviceInfo& d = info[dev];
     if (!d.ok) {
-        hipDeviceProp_t prop;
-        if (hipGetDeviceProperties(&prop, dev) == hipSuccess) {
-            d.cus = prop.multiProcessorCount;
-            d.ok = true;
+        std::lock_guard<std::mutex> lock(g_device_mu);
+        if (!d.ok) {
+            hipDeviceProp_t prop;
+            if (hipGetDeviceProperties(&prop, dev) == hipSuccess) {
+                d.cus = prop.multiProcessorCount;
+                void* h = nullptr;
+                if (hipHostMalloc(&h, 64, hipHostMallocMapped) == hipSuccess && h != nullptr) {
+                    *reinterpret_cast<volatile int*>(h) = 0;
+                    void* dp = nullptr;
+                    if (hipHostGetDevicePointer(&dp, h, 0) == hipSuccess && dp != nullptr) {
+                        d.host_status = reinterpret_cast<int*>(h);
+                        d.host_status_dev = reinterpret_cast<int*>(dp);
+                    } else {
+                        (void)hipHostFree(h);
+                    }
+                }
+                (void)hipGetLastError();
+                d.ok = true;
+            }
         }
     }
     return d;
 }
 
-int env_int(const char* name, int dflt) {
-    const char* v = getenv(name);
-    return v && *v ? atoi(v) : dflt;
+// non-zero: some launch on this device has raised a failure flag since the word was last cleared
+int pending_device_failure() {
+    DeviceInfo& di = device_info();
+    return di.host_status ? *reinterpret_cast<volatile int*>(di.host_status) : 0;
 }
+#define CFPP_REFUSE_AFTER_FAILURE()                          \
+    do {                                                     \
+        if (pending_device_failure()) return CFPP_ERR_DEVICE; \
+    } while (0)
 
 constexpr size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+#ifdef CFPP_TRACE
 long long* g_trace = nullptr;   // see cfpp_debug_set_trace
+#endif
 
 struct WorkspaceLayout {
     size_t qkv_raw, attn_vec, inter, part_ml, part_acc, head_cnt, bar, grp, mbox, team, total;
@@ -1241,10 +1263,38 @@ int launch_stage_c_t(const LayerParams& p, int grid, hipStream_t st) {
     hipLaunchKernelGGL((k_stage_c<NCH, CPD>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
     return launch_check();
 }
+// The one-launch kernels wait for each other's workgroups inside the launch, so every workgroup of the grid has to
+// be resident at the same time.  What the library can establish itself is that the device has room for the grid
+// when nothing else runs on it: the kernel's occupancy (workgroups per compute unit for its registers and LDS) times
+// the compute units.  A grid that does not fit is not launched in one piece; the caller takes the per-stage launches
+// instead.  What it cannot see is other work: kernels of other streams or processes that hold compute units while a
+// one-launch kernel starts can keep some of its workgroups waiting; the bounded waits then expire, the failure flag
+// is raised and the next call on the device reports CFPP_ERR_DEVICE.
+bool one_launch_fits(const void* fn, int block_threads, int grid) {
+    DeviceInfo& di = device_info();
+    int per_cu = 0;
+    {
+        std::lock_guard<std::mutex> lock(g_device_mu);
+        auto it = di.blocks_per_cu.find(fn);
+        if (it != di.blocks_per_cu.end()) per_cu = it->second;
+        else {
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, block_threads, 0) != hipSuccess) {
+                (void)hipGetLastError();
+                per_cu = 0;
+            }
+            di.blocks_per_cu[fn] = per_cu;
+        }
+    }
+    return cfpp_one_launch_fits(grid, di.cus, per_cu) != 0;
+}
+
+template <int NCH, int CPD>
+const void* fused_fn(const LayerParams& p) {
+    return p.H == NCH * kChunk ? (const void*)(k_fused<NCH, CPD, true>) : (const void*)(k_fused<NCH, CPD, false>);
+}
 template <int NCH, int CPD>
 int launch_fused_t(const LayerParams& p, int grid, hipStream_t st) {
-    const void* fn = p.H == NCH * kChunk ? (const void*)(k_fused<NCH, CPD, true>) : (const void*)(k_fused<NCH, CPD, false>);
-    static int coop = env_int("CFPP_COOPERATIVE", 0);
+    const void* fn = fused_fn<NCH, CPD>(p);
     LayerParams pp = p;
     void* args[] = {&pp};
     if (tl_kernel_events) {
@@ -1253,10 +1303,11 @@ int launch_fused_t(const LayerParams& p, int grid, hipStream_t st) {
                                     tl_kernel_events->stop, 0));
         return CFPP_OK;
     }
-    if (coop) CFPP_HIP(hipLaunchCooperativeKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st));
-    else CFPP_HIP(hipLaunchKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st));
+    CFPP_HIP(hipLaunchKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st));
     return CFPP_OK;
 }
+template <int NCH, int CPD>
+bool fused_fits_t(const LayerParams& p, int grid) { return one_launch_fits(fused_fn<NCH, CPD>(p), 2 * kStreamers * 64, grid); }
 
 #define CFPP_NCH_CASES(X) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8)
 // (hidden chunks, MLP-down chunks per streaming wave).  The Pythia family has ffn = 4 hidden, so both
@@ -1284,6 +1335,12 @@ int launch_fused(const Plan& pl, const LayerParams& p, int grid, hipStream_t st)
 #undef X
     return CFPP_ERR_DIMS;
 }
+bool fused_fits(const Plan& pl, const LayerParams& p, int grid) {
+#define X(a, b) if (pl.nch == a && pl.cpd == b) return fused_fits_t<a, b>(p, grid);
+    CFPP_SHAPE_CASES(X)
+#undef X
+    return false;
+}
 template <int NCH>
 int launch_gated_up_t(const LayerParams& p, int grid, hipStream_t st) {
     if (p.H == NCH * kChunk) hipLaunchKernelGGL((k_gated_up<NCH, true>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
@@ -1309,6 +1366,15 @@ int launch_gated_mlp(const Plan& pl, const LayerParams& p, int grid, hipStream_t
 #undef X
     return CFPP_ERR_DIMS;
 }
+bool gated_mlp_fits(const Plan& pl, const LayerParams& p, int grid) {
+#define X(a, b)                                                                                                        \
+    if (pl.nch == a && pl.cpd == b)                                                                                    \
+        return one_launch_fits(p.H == a * kChunk ? (const void*)(k_gated_mlp<a, b, true>) : (const void*)(k_gated_mlp<a, b, false>), \
+                               kStreamers * 64, grid);
+    CFPP_SHAPE_CASES(X)
+#undef X
+    return false;
+}
 
 bool shape_supported(const Plan& pl) {
 #define X(a, b) if (pl.nch == a && pl.cpd == b) return true;
@@ -1322,8 +1388,7 @@ bool shape_supported(const Plan& pl) {
 // workgroups of a streaming launch: one per compute unit
 int streaming_grid() {
     DeviceInfo& di = device_info();
-    const int cus = di.cus > 0 ? di.cus : 256;
-    return cus * env_int("CFPP_WG_PER_CU", 1);
+    return di.cus > 0 ? di.cus : 256;
 }
 
 // workgroups of the fused launch: one per compute unit, all co-resident
@@ -1343,8 +1408,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 // KV splits per head at most: `item_waves` attention waves per workgroup of the fused launch get an item
 int split_cap(int heads, int item_waves) {
-    int ms = env_int("CFPP_MAX_SPLIT", kMaxSplit);
-    ms = ms < 1 ? 1 : (ms > kMaxSplit ? kMaxSplit : ms);
+    int ms = kMaxSplit;
     const int per_head = fused_grid() * item_waves / (heads > 0 ? heads : 1);
     if (ms > per_head) ms = per_head < 1 ? 1 : per_head;
     return ms;
@@ -1363,8 +1427,11 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     if (need_down && (!w->w_down || !w->b_down)) return CFPP_ERR_NULL;
     if (need_out && !io->output) return CFPP_ERR_NULL;
     if (!need_out && (!io->attn_output || !io->mlp_intermediate)) return CFPP_ERR_NULL;
-    if (io->cache_rows < 0) return CFPP_ERR_SEQ;
+    if (io->cache_rows < 0 || io->rope_stride < 0) return CFPP_ERR_SEQ;
+    // a length the host knows is checked here; one in device memory is checked by the kernels (load_seq_len)
     if (!io->d_seq_len && (io->seq_len < 0 || io->seq_len > io->cache_rows)) return CFPP_ERR_SEQ;
+    if (!io->d_seq_len && io->rope_stride > 0 && io->seq_len >= io->cache_rows) return CFPP_ERR_SEQ;
+    if (io->d_seq_len && io->cache_rows < 1) return CFPP_ERR_SEQ;
     const WorkspaceLayout L = workspace_layout(*d);
     if (ws_bytes < L.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CFPP_ERR_WORKSPACE;
     rc = make_plan(*d, plan);
@@ -1390,13 +1457,10 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     // ... and one attention wave per workgroup is better left without an item when the layer has MLP rows: it then
     // carries the MLP-up arrivals of its workgroup (arrival_agents), which gains more than the finer KV split
     // (6.9B at context 2048: TPOT 2.42 instead of 2.49 ms)
-    p.arrival_agents = env_int("CFPP_ARRIVAL_AGENTS", 1);
-    p.max_split = split_cap(d->heads, p.arrival_agents ? kStreamers - 1 : kStreamers);
-    p.row_walk_strided = env_int("CFPP_ROW_WALK_STRIDED", 0);
+    p.arrival_agents = 1;
+    p.max_split = split_cap(d->heads, kStreamers - 1);
     p.norm_rms = 0; p.qkv_head_stride = 3 * d->head_dim; p.qkv_k_off = d->head_dim; p.qkv_v_off = 2 * d->head_dim;
     p.append_kv = 1; p.x_add = nullptr; p.x_sum_out = nullptr; p.c_add_sum = 0;
-    p.dyn_up = env_int("CFPP_DYN_UP", -1);
-    p.qkv_all_waves = env_int("CFPP_QKV_ALL_WAVES", -1);   // -1: decided by the geometry
     char* ws = reinterpret_cast<char*>(workspace);
     p.qkv_raw = reinterpret_cast<float*>(ws + L.qkv_raw);
     p.attn_vec = reinterpret_cast<half_t*>(ws + L.attn_vec);
@@ -1409,7 +1473,10 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     p.mbox = reinterpret_cast<int*>(ws + L.mbox);
     p.team = reinterpret_cast<int*>(ws + L.team);
     p.c_base0 = p.x; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 1;
+    p.host_status = device_info().host_status_dev;
+#ifdef CFPP_TRACE
     p.trace = g_trace;
+#endif
     *out = p;
     return CFPP_OK;
 }
@@ -1419,6 +1486,16 @@ int seq_hint_of(const cfpp_neox_io* io) {
 }
 
 int grid_for_streaming(const Plan&) { return streaming_grid(); }
+
+int run_split(const Plan& pl, LayerParams& p, int seq_hint, hipStream_t st);
+// One layer in the requested mode.  The one-launch kernel is used only when the device can hold its whole grid and
+// every attention wave gets at most one (head, split) item; otherwise the per-stage launches compute the same result.
+int run_layer(const Plan& pl, LayerParams& p, int mode, int seq_hint, hipStream_t st) {
+    if (mode == CFPP_MODE_SPLIT) return run_split(pl, p, seq_hint, st);
+    const int grid = fused_grid();
+    if (p.heads > grid * kStreamers || !fused_fits(pl, p, grid)) return run_split(pl, p, seq_hint, st);
+    return launch_fused(pl, p, grid, st);
+}
 
 int run_split(const Plan& pl, LayerParams& p, int seq_hint, hipStream_t st) {
     const int grid = grid_for_streaming(pl);
@@ -1463,9 +1540,9 @@ int launch_batch_gemv_t(const BatchGemv& a, int grid, hipStream_t st) {
 }
 int launch_batch_mfma(const BatchMfma& a, hipStream_t st) {
     const int grid = a.R / 16;
-    if (env_int("CFPP_BATCH_MFMA_PIPE", 1) && (a.K == 4096 || a.K == 2048)) {
+    if (a.K == 4096 || a.K == 2048) {
         const int wgs = streaming_grid() < grid ? streaming_grid() : grid;
-        const bool one = a.batch <= 16 && env_int("CFPP_BATCH_MFMA_ONE", 1);
+        const bool one = a.batch <= 16;
         if (a.K == 4096) {
             if (one) hipLaunchKernelGGL((k_batch_mfma_pipe<8, true>), dim3(wgs), dim3(512), 0, st, a);
             else hipLaunchKernelGGL((k_batch_mfma_pipe<8, false>), dim3(wgs), dim3(512), 0, st, a);
@@ -1475,12 +1552,8 @@ int launch_batch_mfma(const BatchMfma& a, hipStream_t st) {
         }
         return (int)hipGetLastError();
     }
-    switch (a.K / 256) {
-        case 4: hipLaunchKernelGGL((k_batch_mfma<4>), dim3(grid), dim3(512), 0, st, a); break;
-        case 8: hipLaunchKernelGGL((k_batch_mfma<8>), dim3(grid), dim3(512), 0, st, a); break;
-        case 16: hipLaunchKernelGGL((k_batch_mfma<16>), dim3(grid), dim3(512), 0, st, a); break;
-        default: return CFPP_ERR_DIMS;
-    }
+    if (a.K != 1024) return CFPP_ERR_DIMS;
+    hipLaunchKernelGGL((k_batch_mfma<4>), dim3(grid), dim3(512), 0, st, a);
     return (int)hipGetLastError();
 }
 bool batch_mfma_supported(int rows, int k) { return rows % 16 == 0 && k % 256 == 0 && (k == 1024 || k == 2048 || k == 4096); }
@@ -1543,12 +1616,8 @@ int cfpp_neox_layer_decode(const cfpp_neox_dims* dims, const cfpp_neox_weights* 
     Plan pl;
     int rc = fill_params(dims, w, io, workspace, workspace_bytes, true, true, &p, &pl);
     if (rc) return rc;
-    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    if (mode == CFPP_MODE_SPLIT) return run_split(pl, p, seq_hint_of(io), st);
-    const int grid = fused_grid();
-    // the fused kernel gives every attention wave at most one (head, split) item
-    if (p.heads > grid * kStreamers) return run_split(pl, p, seq_hint_of(io), st);
-    return launch_fused(pl, p, grid, st);
+    CFPP_REFUSE_AFTER_FAILURE();
+    return run_layer(pl, p, mode, seq_hint_of(io), reinterpret_cast<hipStream_t>(stream));
 }
 
 int cfpp_neox_attention_mlp_up(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io,
@@ -1558,6 +1627,7 @@ int cfpp_neox_attention_mlp_up(const cfpp_neox_dims* dims, const cfpp_neox_weigh
     int rc = fill_params(dims, w, io, workspace, workspace_bytes, false, false, &p, &pl);
     if (rc) return rc;
     if (!aligned16(io->attn_output) || !aligned16(io->mlp_intermediate)) return CFPP_ERR_ALIGN;
+    CFPP_REFUSE_AFTER_FAILURE();
     p.inter = reinterpret_cast<half_t*>(io->mlp_intermediate);   // MLP-up writes the caller's tensor directly
     p.out = reinterpret_cast<half_t*>(io->attn_output);          // stage C: W_o attn + b_o only
     p.c_base0 = nullptr; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 0;
@@ -1586,11 +1656,13 @@ int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_
     }
     if (a->residual && !aligned16(a->residual)) return CFPP_ERR_ALIGN;
     if (a->seq_len < 0) return CFPP_ERR_SEQ;
+    if (a->mode != CFPP_MODE_FUSED && a->mode != CFPP_MODE_SPLIT) return CFPP_ERR_MODE;
     const WorkspaceLayout L = workspace_layout(d);
     if (workspace_bytes < L.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CFPP_ERR_WORKSPACE;
     Plan pl;
     if ((rc = make_plan(d, &pl))) return rc;
     if (!shape_supported(pl)) return CFPP_ERR_DIMS;
+    CFPP_REFUSE_AFTER_FAILURE();
 
     // start from the NeoX parameter block of the same geometry, then switch the family-specific parts
     cfpp_neox_weights w{};
@@ -1603,21 +1675,20 @@ int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_
     LayerParams p;
     if ((rc = fill_params(&d, &w, &io, workspace, workspace_bytes, true, true, &p, &pl))) return rc;
     p.F = 0;                                     // no MLP rows in stage A
+    p.arrival_agents = 0;
     p.max_split = split_cap(d.heads, kStreamers);    // ... so no attention wave is kept free for MLP-up arrivals
     p.ln_b = nullptr; p.ln2_w = nullptr; p.ln2_b = nullptr; p.b_qkv = nullptr; p.b_o = nullptr;
     p.w_up = nullptr; p.b_up = nullptr; p.w_down = nullptr; p.b_down = nullptr;
     p.norm_rms = 1;
     p.qkv_head_stride = d.head_dim; p.qkv_k_off = d.hidden; p.qkv_v_off = 2 * d.hidden;
     p.append_kv = 0;
+    p.rope_half_table = 1;                       // cos / sin hold the D/2 pair angles
     p.x_add = reinterpret_cast<const half_t*>(a->residual);
     p.x_sum_out = reinterpret_cast<half_t*>(a->residual);
     p.c_base0 = nullptr; p.c_base1 = nullptr; p.c_use_o = 1; p.c_use_down = 0;
     p.c_add_sum = a->add_residual ? 1 : 0;
-    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const int grid = fused_grid();
-    if (env_int("CFPP_LLAMA_SPLIT", 0) || p.heads > grid * kStreamers) return run_split(pl, p, a->seq_len, st);
-    // one launch: the attention waves fetch their K/V tiles while the streaming waves do the QKV rows
-    return launch_fused(pl, p, grid, st);
+    // one launch (the attention waves fetch their K/V tiles while the streaming waves do the QKV rows) or one per stage
+    return run_layer(pl, p, a->mode, a->seq_len, reinterpret_cast<hipStream_t>(stream));
 }
 
 // The reference's plain llama_decoder_layer op: as cfpp_llama_attention_decode without a residual, with weights stored
@@ -1640,7 +1711,7 @@ int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t
         if (!q) return CFPP_ERR_NULL;
         if (!aligned16(q)) return CFPP_ERR_ALIGN;
     }
-    if (a->residual != nullptr || a->add_residual) return CFPP_ERR_MODE;      // this op has no residual stream
+    if (a->residual != nullptr || a->add_residual || a->mode != CFPP_MODE_FUSED) return CFPP_ERR_MODE;      // no residual stream, one variant
     if (a->seq_len < 0) return CFPP_ERR_SEQ;
     const size_t need = cfpp_llama_plain_workspace_bytes(a->hidden, a->heads, a->head_dim);
     if (need == 0) return CFPP_ERR_DIMS;
@@ -1659,13 +1730,8 @@ int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t
     half_t* xn = reinterpret_cast<half_t*>(reinterpret_cast<char*>(cnt) + align_up((size_t)3 * ppm * 4, 256));
     auto h = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
 
-    const bool norm_inside = env_int("CFPP_PLAIN_NORM_INSIDE", 1) != 0;
-    if (!norm_inside) {
-        BatchNorm n{};
-        n.x = h(a->input); n.x_add = nullptr; n.norm_w = h(a->rms_w); n.sum_out = nullptr; n.y = xn;
-        n.eps = a->eps; n.K = H; n.batch = 1;
-        if ((rc = launch_batch_norm(pl.nch, n, st))) return rc;
-    }
+    (void)xn;
+    CFPP_REFUSE_AFTER_FAILURE();
 
     cfpp_neox_weights w{};
     w.ln_w = a->rms_w; w.ln_b = a->rms_w; w.w_qkv = a->w_qkv; w.b_qkv = a->rms_w; w.w_o = a->w_o; w.b_o = a->rms_w;
@@ -1677,6 +1743,7 @@ int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t
     LayerParams p;
     if ((rc = fill_params(&d, &w, &io, workspace, workspace_bytes, true, true, &p, &pl))) return rc;
     p.F = 0;
+    p.arrival_agents = 0;
     p.max_split = split_cap(d.heads, kStreamers);
     p.qkv_head_stride = d.head_dim; p.qkv_k_off = H; p.qkv_v_off = 2 * H;
     p.append_kv = 0;
@@ -1690,9 +1757,8 @@ int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t
         hipLaunchKernelGGL(k_gemv_t, dim3(panels * g.slices), dim3(kStreamers * 64), 0, st, g);
         return (int)hipGetLastError();
     };
-    // the QKV launch normalises the input row on its way in
-    if ((rc = norm_inside ? gemv(h(a->w_qkv), 3, h(a->input), h(a->rms_w), p.qkv_raw, nullptr)
-                          : gemv(h(a->w_qkv), 3, xn, nullptr, p.qkv_raw, nullptr))) return rc;
+    // the QKV launch normalises the input row on its way in (a separate norm launch was measured slower)
+    if ((rc = gemv(h(a->w_qkv), 3, h(a->input), h(a->rms_w), p.qkv_raw, nullptr))) return rc;
     const int bgrid = (p.heads * split_bound(a->seq_len, p.max_split) + kStreamers - 1) / kStreamers;
     hipLaunchKernelGGL(k_stage_b_pairs, dim3(bgrid), dim3(kStreamers * 64), 0, st, p);
     if ((rc = (int)hipGetLastError())) return rc;
@@ -1709,6 +1775,7 @@ int cfpp_llama_mlp(const cfpp_llama_mlp_args* m, void* workspace, size_t workspa
     if (!m || !workspace) return CFPP_ERR_NULL;
     const size_t need = cfpp_llama_mlp_workspace_bytes(m->hidden, m->ffn);
     if (need == 0 || !(m->eps > 0.f)) return CFPP_ERR_DIMS;
+    if (m->mode != CFPP_MODE_FUSED && m->mode != CFPP_MODE_SPLIT) return CFPP_ERR_MODE;
     if (workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CFPP_ERR_WORKSPACE;
     const void* req[] = {m->rms_w, m->w_gate_up, m->w_down, m->input, m->output};
     for (const void* q : req) {
@@ -1727,15 +1794,16 @@ int cfpp_llama_mlp(const cfpp_llama_mlp_args* m, void* workspace, size_t workspa
     p.inter = reinterpret_cast<half_t*>(workspace);
     p.out = reinterpret_cast<half_t*>(m->output);
     p.c_base0 = p.x; p.c_use_o = 0; p.c_use_down = 1;
+    p.host_status = device_info().host_status_dev;
+    CFPP_REFUSE_AFTER_FAILURE();
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    if (env_int("CFPP_LLAMA_MLP_FUSED", 1)) {
-        // one launch: the down rows wait for the phases of the intermediate inside the kernel
-        char* ws = reinterpret_cast<char*>(workspace) + align_up((size_t)m->ffn * 2, 256);
-        p.bar = reinterpret_cast<int*>(ws);
-        p.grp = reinterpret_cast<int*>(ws + 256);
-        p.mbox = reinterpret_cast<int*>(ws + 256 + align_up((size_t)(kBarExit + 1) * kEventGroups * kMailboxInts * 4, 256));
-        return launch_gated_mlp(pl, p, fused_grid(), st);
-    }
+    char* ws = reinterpret_cast<char*>(workspace) + align_up((size_t)m->ffn * 2, 256);
+    p.bar = reinterpret_cast<int*>(ws);
+    p.grp = reinterpret_cast<int*>(ws + 256);
+    p.mbox = reinterpret_cast<int*>(ws + 256 + align_up((size_t)(kBarExit + 1) * kEventGroups * kMailboxInts * 4, 256));
+    // one launch (the down rows wait for the phases of the intermediate inside the kernel) when the device holds the
+    // whole grid; two launches (gate/up rows, down rows) otherwise or on request
+    if (m->mode == CFPP_MODE_FUSED && gated_mlp_fits(pl, p, fused_grid())) return launch_gated_mlp(pl, p, fused_grid(), st);
     const int grid = streaming_grid();
     int rc = launch_gated_up(pl, p, grid, st);
     if (rc) return rc;
@@ -1768,7 +1836,7 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
     const int nch = (d.hidden + kChunk - 1) / kChunk;
     // two workgroups per compute unit for the row streams: a second wave per SIMD covers the latencies of the
     // per-sequence reductions
-    const int grid = streaming_grid() * env_int("CFPP_BATCH_WGS_PER_CU", 2);
+    const int grid = streaming_grid() * 2;
     const int waves = grid * kStreamers;
     if (grid < 1 || (3 * d.hidden + waves - 1) / waves + 2 > kBatchParkRows) return CFPP_ERR_DIMS;
     char* ws = reinterpret_cast<char*>(workspace);
@@ -1777,7 +1845,8 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
 
     // matrix-core kernels where the geometry allows (and from two sequences on: a single sequence is served as
     // well by the dot-instruction kernel, without the separate norm launch)
-    const bool mfma = batch_mfma_supported(d.hidden, d.hidden) && a->batch >= env_int("CFPP_BATCH_MFMA_FROM", 2);
+    const bool mfma = batch_mfma_supported(d.hidden, d.hidden) && a->batch >= 2;
+    CFPP_REFUSE_AFTER_FAILURE();
     if (mfma) {
         BatchNorm n{};
         n.x = h(a->input); n.x_add = h(a->residual); n.norm_w = h(a->rms_w);
@@ -1810,13 +1879,14 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
     p.part_acc = reinterpret_cast<float*>(ws + L.part_acc);
     p.head_cnt = reinterpret_cast<int*>(ws + L.head_cnt);
     p.bar = reinterpret_cast<int*>(ws + L.bar);
+    p.host_status = device_info().host_status_dev;
     p.qkv_head_stride = d.head_dim; p.qkv_k_off = d.hidden; p.qkv_v_off = 2 * d.hidden;
     p.append_kv = 1;
+    p.rope_half_table = 1;                       // a cos_sin row holds the D/2 pair angles' cosines, then their sines
     // enough (sequence, head, split) items to fill the attention waves about twice, and no more
     int ms = (2 * streaming_grid() * kStreamers) / (a->batch * d.heads);
     ms = ms < 1 ? 1 : (ms > 32 ? 32 : ms);
-    p.max_split = env_int("CFPP_MAX_SPLIT", ms);
-    if (p.max_split < 1 || p.max_split > kMaxSplit) return CFPP_ERR_DIMS;
+    p.max_split = ms;
     BatchAttn b{};
     b.batch = a->batch; b.layer_id = a->layer_id;
     b.indptr = a->paged_kv_indptr; b.indices = a->paged_kv_indices;
@@ -1887,10 +1957,28 @@ int cfpp_workspace_check(const cfpp_neox_dims* dims, void* workspace, void* stre
     return CFPP_OK;
 }
 
+int cfpp_device_status(int clear) {
+    DeviceInfo& di = device_info();
+    if (!di.host_status) return 0;
+    volatile int* w = reinterpret_cast<volatile int*>(di.host_status);
+    const int flags = *w;
+    if (clear) *w = 0;
+    return flags;
+}
+
+int cfpp_one_launch_fits(int grid, int compute_units, int blocks_per_cu) {
+    if (grid < 1 || compute_units < 1 || blocks_per_cu < 1) return 0;
+    return (long long)grid <= (long long)compute_units * blocks_per_cu ? 1 : 0;
+}
+
+#ifdef CFPP_TRACE
+// Profiling builds only (not declared in cfpp.h): when set to a device buffer of [workgroups][16 waves][16 slots]
+// int64, every fused launch stores 100 MHz timestamps of its phase boundaries there; NULL switches it off.
 int cfpp_debug_set_trace(void* device_buffer) {
     g_trace = reinterpret_cast<long long*>(device_buffer);
     return CFPP_OK;
 }
+#endif
 
 // ---- per-layer contexts --------------------------------------------------------------------------
 namespace {
@@ -1975,6 +2063,17 @@ int cfpp_ctx_step(int family, int64_t id, const cfpp_neox_weights* w, const cfpp
     return cfpp_neox_layer_decode(&c.dims, &ww, &ii, mode, c.ws, c.ws_bytes, stream);
 }
 
+int cfpp_ctx_check(int family, int64_t id, void* stream) {
+    Ctx c;
+    {
+        std::lock_guard<std::mutex> lock(g_ctx_mu);
+        auto it = g_ctx.find(std::make_pair(family, id));
+        if (it == g_ctx.end()) return CFPP_ERR_CONTEXT;
+        c = it->second;
+    }
+    return cfpp_workspace_check(&c.dims, c.ws, stream);
+}
+
 int cfpp_ctx_destroy(int family, int64_t id) {
     std::lock_guard<std::mutex> lock(g_ctx_mu);
     auto it = g_ctx.find(std::make_pair(family, id));
@@ -2035,6 +2134,9 @@ struct cfpp_neox_stack {
     int hist_cap = 0;
     void* ws = nullptr;
     size_t ws_bytes = 0;
+    // the device-resident position changes only through set_state and the steps, all of which pass through the host:
+    // this mirror lets the host refuse steps that would run past the caches (-1: not set yet)
+    long long host_seq_len = -1;
     hipStream_t own_stream = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
@@ -2059,17 +2161,13 @@ cfpp_neox_io stack_layer_io(const cfpp_neox_stack* s, int l) {
 }
 int stack_enqueue_layer(cfpp_neox_stack* s, int l, hipStream_t st) {
     const cfpp_neox_io io = stack_layer_io(s, l);
-    if (s->desc.mode != CFPP_MODE_FUSED || !env_int("CFPP_STACK_TAGS", 1))
-        return cfpp_neox_layer_decode(&s->desc.dims, &s->layers[l], &io, s->desc.mode, s->ws, s->ws_bytes, st);
     LayerParams p;
     Plan pl;
     int rc = fill_params(&s->desc.dims, &s->layers[l], &io, s->ws, s->ws_bytes, true, true, &p, &pl);
     if (rc) return rc;
-    const int grid = fused_grid();
-    if (p.heads > grid * kStreamers) return run_split(pl, p, seq_hint_of(&io), st);
     // launch tags from the stack's step counter: no launch has to publish a generation for the next one
     p.tag_src = s->state + 3; p.tag_mul = s->desc.n_layers; p.tag_add = l;
-    return launch_fused(pl, p, grid, st);
+    return run_layer(pl, p, s->desc.mode, seq_hint_of(&io), st);
 }
 
 int stack_enqueue_step(cfpp_neox_stack* s, hipStream_t st) {
@@ -2142,20 +2240,44 @@ int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out) {
 
 int cfpp_stack_set_state(cfpp_neox_stack* s, int32_t token, int32_t seq_len, void* stream) {
     if (!s) return CFPP_ERR_NULL;
-    if (seq_len < 0 || seq_len > s->desc.cache_rows) return CFPP_ERR_SEQ;
+    if (seq_len < 0 || seq_len >= s->desc.cache_rows) return CFPP_ERR_SEQ;     // the next step appends row seq_len
     if (token < 0 || token >= s->desc.vocab) return CFPP_ERR_DIMS;
     hipLaunchKernelGGL(k_set_state, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(stream), s->state, token, seq_len);
-    return launch_check();
+    const int rc = launch_check();
+    if (!rc) s->host_seq_len = seq_len;
+    return rc;
 }
+
+namespace {
+// `n` more steps need cache rows host_seq_len .. host_seq_len + n - 1
+int stack_room(const cfpp_neox_stack* s, long long n) {
+    const long long at = s->host_seq_len < 0 ? 0 : s->host_seq_len;
+    return at + n <= (long long)s->desc.cache_rows ? CFPP_OK : CFPP_ERR_SEQ;
+}
+void stack_advance(cfpp_neox_stack* s, long long n) { s->host_seq_len = (s->host_seq_len < 0 ? 0 : s->host_seq_len) + n; }
+}  // namespace
 
 int cfpp_stack_step(cfpp_neox_stack* s, void* stream) {
     if (!s) return CFPP_ERR_NULL;
-    return stack_enqueue_step(s, reinterpret_cast<hipStream_t>(stream));
+    int rc = stack_room(s, 1);
+    if (rc) return rc;
+    CFPP_REFUSE_AFTER_FAILURE();
+    rc = stack_enqueue_step(s, reinterpret_cast<hipStream_t>(stream));
+    if (!rc) stack_advance(s, 1);
+    return rc;
+}
+
+int cfpp_stack_check(cfpp_neox_stack* s, void* stream) {
+    if (!s) return CFPP_ERR_NULL;
+    return cfpp_workspace_check(&s->desc.dims, s->ws, stream);
 }
 
 int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream) {
     if (!s) return CFPP_ERR_NULL;
     if (n_steps < 0) return CFPP_ERR_DIMS;
+    int room = stack_room(s, n_steps);
+    if (room) return room;
+    CFPP_REFUSE_AFTER_FAILURE();
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (!st) {
         if (!s->own_stream) CFPP_HIP(hipStreamCreateWithFlags(&s->own_stream, hipStreamDefault));   // ordered with the null stream
@@ -2171,20 +2293,35 @@ int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream) {
         s->graph = g;
         CFPP_HIP(hipGraphInstantiate(&s->exec, s->graph, nullptr, nullptr, 0));
     }
-    for (int i = 0; i < n_steps; ++i) CFPP_HIP(hipGraphLaunch(s->exec, st));
+    for (int i = 0; i < n_steps; ++i) {
+        CFPP_HIP(hipGraphLaunch(s->exec, st));
+        stack_advance(s, 1);
+    }
     if (!stream) CFPP_HIP(hipStreamSynchronize(st));
     return CFPP_OK;
 }
 
 int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, float* lm_head_ms, float* total_ms) {
     if (!s) return CFPP_ERR_NULL;
+    {
+        const int room = stack_room(s, 1);
+        if (room) return room;
+    }
+    CFPP_REFUSE_AFTER_FAILURE();
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const int L = s->desc.n_layers;
     std::vector<hipEvent_t> ev(L + 3);
     for (auto& e : ev) CFPP_HIP(hipEventCreate(&e));
     // fused mode: one kernel per layer, timed from its own start to its own end; split mode (three kernels per layer):
     // stream events between the layers, which include the launch gaps
-    const bool fused = s->desc.mode == CFPP_MODE_FUSED && s->desc.dims.heads <= fused_grid() * kStreamers;
+    bool fused = false;
+    if (s->desc.mode == CFPP_MODE_FUSED && s->desc.dims.heads <= fused_grid() * kStreamers) {
+        const cfpp_neox_io io0 = stack_layer_io(s, 0);
+        LayerParams p0;
+        Plan pl0;
+        if (fill_params(&s->desc.dims, &s->layers[0], &io0, s->ws, s->ws_bytes, true, true, &p0, &pl0) == CFPP_OK)
+            fused = fused_fits(pl0, p0, fused_grid());
+    }
     std::vector<KernelEvents> kev(fused ? L : 0);
     for (auto& k : kev) {
         CFPP_HIP(hipEventCreate(&k.start));
@@ -2233,6 +2370,7 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
     for (auto& e : ev) (void)hipEventDestroy(e);
     for (auto& k : kev) { (void)hipEventDestroy(k.start); (void)hipEventDestroy(k.stop); }
     (void)hipEventDestroy(end);
+    if (!rc) stack_advance(s, 1);
     return rc;
 }
 

@@ -14,6 +14,8 @@
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
+#include <dlfcn.h>
+
 #include <map>
 #include <memory>
 #include <mutex>
@@ -34,7 +36,30 @@ struct Model {
 const Model kPythia2b8{"pythia_2b8", 0, {2560, 32, 80, 20, 10240, 1e-5f}};
 const Model kPythia6b9{"pythia_6b9", 1, {4096, 32, 128, 32, 16384, 1e-5f}};
 
+// Scratch buffers handed to the C ABI, one per (device, stream, geometry): calls on one stream are ordered, so they
+// can share one.  Zero-initialised; the kernels leave their counters at zero after every call.
+struct ScratchKey {
+    int device; void* stream; int kind; int a, b, c, d;
+    bool operator<(const ScratchKey& o) const {
+        return std::tie(device, stream, kind, a, b, c, d) < std::tie(o.device, o.stream, o.kind, o.a, o.b, o.c, o.d);
+    }
+};
+std::mutex g_scratch_mu;
+std::map<ScratchKey, torch::Tensor> g_scratch;
+
 void check_rc(int rc, const char* what) {
+    if (rc == CFPP_ERR_DEVICE) {
+        // a launch on this device has raised a failure flag: report it once, clear it, and drop the scratch buffers
+        // (an expired wait leaves counters mid-flight; new buffers start from zero)
+        const int flags = cfpp_device_status(1);
+        {
+            std::lock_guard<std::mutex> lock(g_scratch_mu);
+            g_scratch.clear();
+        }
+        TORCH_CHECK(false, what, ": ", cfpp_status_str(rc), " (flags ", flags,
+                    ": 1 = a bounded device-side wait expired, is other work running on the GPU?; 2 = a device-side "
+                    "current_seq_len was out of range); results since the last successful check are invalid");
+    }
     TORCH_CHECK(rc == 0, what, ": ", cfpp_status_str(rc), " (status ", rc, ")");
 }
 
@@ -62,23 +87,28 @@ int64_t check_cache(const Tensor& t, const char* name, int64_t H, const Tensor& 
     return t.size(0);
 }
 
-// one zero-initialised scratch buffer per (device, stream): calls on one stream are ordered, so they can share
-Tensor workspace_for(const cfpp_neox_dims& d, const torch::Device& dev, hipStream_t st) {
-    static std::mutex mu;
-    static std::map<std::tuple<int, void*, int, int>, Tensor> cache;
-    std::lock_guard<std::mutex> lock(mu);
-    auto key = std::make_tuple((int)dev.index(), (void*)st, (int)d.hidden, (int)d.ffn);
-    auto it = cache.find(key);
-    if (it != cache.end()) return it->second;
-    const int64_t bytes = (int64_t)cfpp_neox_workspace_bytes(&d);
+Tensor scratch_for(const ScratchKey& key, int64_t bytes, const torch::Device& dev) {
     TORCH_CHECK(bytes > 0, "unsupported layer dimensions");
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    auto it = g_scratch.find(key);
+    if (it != g_scratch.end() && it->second.numel() >= bytes + 256) return it->second;
     Tensor ws = torch::zeros({bytes + 256}, torch::TensorOptions().dtype(torch::kUInt8).device(dev));
-    cache[key] = ws;
+    g_scratch[key] = ws;
     return ws;
+}
+// The layout of a layer workspace depends on every dimension but the rotary one, so all of them are in the key: a
+// buffer is never reused under another layout (its counters would sit on stale data).
+Tensor workspace_for(const cfpp_neox_dims& d, const torch::Device& dev, hipStream_t st) {
+    return scratch_for(ScratchKey{(int)dev.index(), (void*)st, 0, d.hidden, d.heads, d.head_dim, d.ffn},
+                       (int64_t)cfpp_neox_workspace_bytes(&d), dev);
 }
 void* ws_ptr(const Tensor& ws) {
     auto p = reinterpret_cast<uintptr_t>(ws.data_ptr());
     return reinterpret_cast<void*>((p + 255) / 256 * 256);
+}
+// bytes of the tensor that remain behind the aligned pointer: what the C ABI checks its needs against
+size_t ws_capacity(const Tensor& ws) {
+    return (size_t)ws.numel() - (size_t)(reinterpret_cast<uintptr_t>(ws_ptr(ws)) - reinterpret_cast<uintptr_t>(ws.data_ptr()));
 }
 
 struct LayerArgs {
@@ -144,7 +174,7 @@ std::tuple<Tensor, Tensor, Tensor> decoder_layer(const Model& m, int mode, const
     io.output = out.data_ptr(); io.k_new = k.data_ptr(); io.v_new = v.data_ptr();
     hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     Tensor ws = workspace_for(d, a.input.device(), st);
-    check_rc(cfpp_neox_layer_decode(&d, &w, &io, mode, ws_ptr(ws), cfpp_neox_workspace_bytes(&d), st), m.name);
+    check_rc(cfpp_neox_layer_decode(&d, &w, &io, mode, ws_ptr(ws), ws_capacity(ws), st), m.name);
     return std::make_tuple(out, k, v);
 }
 
@@ -164,7 +194,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> attention_only(const Model& m, const 
     io.k_new = k.data_ptr(); io.v_new = v.data_ptr();
     hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     Tensor ws = workspace_for(d, a.input.device(), st);
-    check_rc(cfpp_neox_attention_mlp_up(&d, &w, &io, ws_ptr(ws), cfpp_neox_workspace_bytes(&d), st), m.name);
+    check_rc(cfpp_neox_attention_mlp_up(&d, &w, &io, ws_ptr(ws), ws_capacity(ws), st), m.name);
     return std::make_tuple(attn, inter, k, v);
 }
 
@@ -276,11 +306,22 @@ std::tuple<Tensor, Tensor, Tensor> graph_decode_step(const Model& m, int64_t id,
 }
 
 void destroy_graph_context(const Model& m, int64_t id) {
+    bool known = false;
+    torch::Device dev{torch::kCPU};
     {
         std::lock_guard<std::mutex> lock(g_mu);
-        g_ctx.erase(std::make_pair(m.family, id));
+        auto it = g_ctx.find(std::make_pair(m.family, id));
+        if (it != g_ctx.end()) { known = true; dev = it->second.k_cache.device(); g_ctx.erase(it); }
+    }
+    // the last chance to learn that a step of this context failed on the device (an expired wait, a device-side
+    // current_seq_len out of range): read its status word before the buffers go
+    int status = CFPP_OK;
+    if (known) {
+        c10::hip::HIPGuardMasqueradingAsCUDA guard(dev);
+        status = cfpp_ctx_check(m.family, id, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
     }
     check_rc(cfpp_ctx_destroy(m.family, id), "destroy_graph_context");
+    check_rc(status, "destroy_graph_context (steps of this context)");
 }
 
 // ---- whole-model decode (our counterpart of the reference's Python decode loop) --------------------
@@ -397,7 +438,7 @@ const Model& kpythia_6b9 = kPythia6b9;
 std::tuple<Tensor, Tensor, Tensor> llama_attention_impl(const char* op, Tensor input, c10::optional<Tensor> residual_opt,
                                                         Tensor weight_qkv, Tensor weight_o, Tensor k_cache, Tensor v_cache,
                                                         Tensor rms_input_weight, double eps, Tensor cos, Tensor sin,
-                                                        int64_t num_heads, bool add_residual) {
+                                                        int64_t num_heads, bool add_residual, bool split) {
     TORCH_CHECK(input.defined() && input.dim() >= 1, "input is undefined");
     const int64_t H = input.numel();
     TORCH_CHECK(num_heads > 0 && H % num_heads == 0, "hidden size ", H, " is not a multiple of num_heads ", num_heads);
@@ -422,6 +463,7 @@ std::tuple<Tensor, Tensor, Tensor> llama_attention_impl(const char* op, Tensor i
     a.rms_w = rms_input_weight.data_ptr(); a.w_qkv = weight_qkv.data_ptr(); a.w_o = weight_o.data_ptr();
     a.input = input.data_ptr(); a.residual = residual_opt.has_value() ? residual_opt->data_ptr() : nullptr; a.output = out.data_ptr();
     a.add_residual = add_residual ? 1 : 0;
+    a.mode = split ? CFPP_MODE_SPLIT : CFPP_MODE_FUSED;
     a.k_new = k.data_ptr(); a.v_new = v.data_ptr();
     // an empty cache has no storage: any valid pointer will do, no row of it is read
     a.k_cache = rows_k > 0 ? k_cache.data_ptr() : input.data_ptr();
@@ -433,16 +475,16 @@ std::tuple<Tensor, Tensor, Tensor> llama_attention_impl(const char* op, Tensor i
     hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     const cfpp_neox_dims d{a.hidden, a.heads, a.head_dim, a.head_dim, 4 * a.hidden, a.eps};
     Tensor ws = workspace_for(d, input.device(), st);
-    check_rc(cfpp_llama_attention_decode(&a, ws_ptr(ws), bytes, st), op);
+    check_rc(cfpp_llama_attention_decode(&a, ws_ptr(ws), ws_capacity(ws), st), op);
     return std::make_tuple(out, k, v);
 }
 
 std::tuple<Tensor, Tensor, Tensor, Tensor> llama_decoder_layer_sglang(Tensor input, Tensor residual, Tensor weight_qkv,
                                                                       Tensor weight_o, Tensor k_cache, Tensor v_cache,
                                                                       Tensor rms_input_weight, double eps, Tensor cos, Tensor sin,
-                                                                      int64_t num_heads) {
+                                                                      int64_t num_heads, bool split) {
     auto r = llama_attention_impl("llama_decoder_layer_sglang", input, residual, weight_qkv, weight_o, k_cache, v_cache,
-                                  rms_input_weight, eps, cos, sin, num_heads, false);
+                                  rms_input_weight, eps, cos, sin, num_heads, false, split);
     return std::make_tuple(std::get<0>(r), residual, std::get<1>(r), std::get<2>(r));
 }
 
@@ -476,6 +518,7 @@ std::tuple<Tensor, Tensor, Tensor> llama_decoder_layer(Tensor input, Tensor weig
     a.hidden = (int32_t)H; a.heads = (int32_t)num_heads; a.head_dim = (int32_t)D; a.eps = 1e-6f;
     a.rms_w = rms_input_weight.data_ptr(); a.w_qkv = weight_qkv.data_ptr(); a.w_o = weight_o.data_ptr();
     a.input = input.data_ptr(); a.residual = nullptr; a.output = out.data_ptr(); a.add_residual = 0;
+    a.mode = CFPP_MODE_FUSED;
     a.k_new = k.data_ptr(); a.v_new = v.data_ptr();
     a.k_cache = rows_k > 0 ? k_cache.data_ptr() : input.data_ptr();
     a.v_cache = rows_k > 0 ? v_cache.data_ptr() : input.data_ptr();
@@ -484,21 +527,9 @@ std::tuple<Tensor, Tensor, Tensor> llama_decoder_layer(Tensor input, Tensor weig
     const size_t bytes = cfpp_llama_plain_workspace_bytes(a.hidden, a.heads, a.head_dim);
     TORCH_CHECK(bytes > 0, "unsupported layer dimensions (hidden ", H, ", heads ", num_heads, ")");
     hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
-    static std::mutex mu;
-    static std::map<std::tuple<int, void*, int, int>, Tensor> cache;
-    Tensor ws;
-    {
-        std::lock_guard<std::mutex> lock(mu);
-        auto key = std::make_tuple((int)input.device().index(), (void*)st, (int)H, (int)D);
-        auto it = cache.find(key);
-        if (it == cache.end()) {
-            ws = torch::zeros({(int64_t)bytes + 256}, torch::TensorOptions().dtype(torch::kUInt8).device(input.device()));
-            cache[key] = ws;
-        } else {
-            ws = it->second;
-        }
-    }
-    check_rc(cfpp_llama_attention_plain(&a, ws_ptr(ws), bytes, st), op);
+    Tensor ws = scratch_for(ScratchKey{(int)input.device().index(), (void*)st, 1, (int)H, (int)num_heads, (int)D, 0}, (int64_t)bytes,
+                            input.device());
+    check_rc(cfpp_llama_attention_plain(&a, ws_ptr(ws), ws_capacity(ws), st), op);
     return std::make_tuple(out, k, v);
 }
 
@@ -554,26 +585,13 @@ void llama_decoder_layer_batch_decode_sglang(Tensor output, Tensor residual_outp
     const size_t bytes = cfpp_llama_batch_workspace_bytes(a.hidden, a.heads, a.head_dim, a.batch);
     TORCH_CHECK(bytes > 0, "unsupported layer dimensions (hidden ", H, ", head size ", D, ")");
     hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
-    // zero-initialised scratch per (device, stream, geometry, batch): its counters return to zero after every call
-    static std::mutex mu;
-    static std::map<std::tuple<int, void*, int, int, int>, Tensor> cache;
-    Tensor ws;
-    {
-        std::lock_guard<std::mutex> lock(mu);
-        auto key = std::make_tuple((int)input.device().index(), (void*)st, (int)H, (int)D, (int)B);
-        auto it = cache.find(key);
-        if (it == cache.end()) {
-            ws = torch::zeros({(int64_t)bytes + 256}, torch::TensorOptions().dtype(torch::kUInt8).device(input.device()));
-            cache[key] = ws;
-        } else {
-            ws = it->second;
-        }
-    }
-    check_rc(cfpp_llama_batch_decode(&a, ws_ptr(ws), bytes, st), op);
+    Tensor ws = scratch_for(ScratchKey{(int)input.device().index(), (void*)st, 2, (int)H, (int)(H / D), (int)D, (int)B}, (int64_t)bytes,
+                            input.device());
+    check_rc(cfpp_llama_batch_decode(&a, ws_ptr(ws), ws_capacity(ws), st), op);
 }
 
 // output = input + W_down (silu(Wg n) * (Wu n)), n = RMSNorm(input) * rms_weight; gate_up_weight = [Wg; Wu] ([2F, H])
-Tensor llama_mlp(Tensor input, Tensor rms_weight, Tensor gate_up_weight, Tensor down_weight, double eps) {
+Tensor llama_mlp(Tensor input, Tensor rms_weight, Tensor gate_up_weight, Tensor down_weight, double eps, bool split) {
     TORCH_CHECK(input.defined() && input.dim() >= 1, "input is undefined");
     const int64_t H = input.numel();
     check_half(input, "input", H, input);
@@ -589,25 +607,12 @@ Tensor llama_mlp(Tensor input, Tensor rms_weight, Tensor gate_up_weight, Tensor 
     m.hidden = (int32_t)H; m.ffn = (int32_t)F; m.eps = (float)eps;
     m.rms_w = rms_weight.data_ptr(); m.w_gate_up = gate_up_weight.data_ptr(); m.w_down = down_weight.data_ptr();
     m.input = input.data_ptr(); m.output = out.data_ptr();
+    m.mode = split ? CFPP_MODE_SPLIT : CFPP_MODE_FUSED;
     const size_t bytes = cfpp_llama_mlp_workspace_bytes(m.hidden, m.ffn);
     TORCH_CHECK(bytes > 0, "unsupported MLP dimensions (hidden ", H, ", ffn ", F, ")");
     hipStream_t st = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
-    // zero-initialised scratch per (device, stream, geometry): its counters return to zero after every call
-    static std::mutex mu;
-    static std::map<std::tuple<int, void*, int, int>, Tensor> cache;
-    Tensor ws;
-    {
-        std::lock_guard<std::mutex> lock(mu);
-        auto key = std::make_tuple((int)input.device().index(), (void*)st, (int)H, (int)F);
-        auto it = cache.find(key);
-        if (it == cache.end()) {
-            ws = torch::zeros({(int64_t)bytes + 256}, input.options().dtype(torch::kUInt8));
-            cache[key] = ws;
-        } else {
-            ws = it->second;
-        }
-    }
-    check_rc(cfpp_llama_mlp(&m, ws_ptr(ws), bytes, st), "llama_mlp");
+    Tensor ws = scratch_for(ScratchKey{(int)input.device().index(), (void*)st, 3, (int)H, (int)F, 0, 0}, (int64_t)bytes, input.device());
+    check_rc(cfpp_llama_mlp(&m, ws_ptr(ws), ws_capacity(ws), st), "llama_mlp");
     return out;
 }
 
@@ -616,10 +621,10 @@ Tensor llama_mlp(Tensor input, Tensor rms_weight, Tensor gate_up_weight, Tensor 
 std::tuple<Tensor, Tensor, Tensor> llama_decoder_layer_full(Tensor input, Tensor weight_qkv, Tensor weight_o, Tensor k_cache,
                                                             Tensor v_cache, Tensor rms_input_weight, Tensor rms_post_weight,
                                                             Tensor gate_up_weight, Tensor down_weight, double eps, Tensor cos,
-                                                            Tensor sin, int64_t num_heads) {
+                                                            Tensor sin, int64_t num_heads, bool split) {
     auto r = llama_attention_impl("llama_decoder_layer_full", input, c10::nullopt, weight_qkv, weight_o, k_cache, v_cache,
-                                  rms_input_weight, eps, cos, sin, num_heads, true);
-    Tensor out = llama_mlp(std::get<0>(r), rms_post_weight, gate_up_weight, down_weight, eps);
+                                  rms_input_weight, eps, cos, sin, num_heads, true, split);
+    Tensor out = llama_mlp(std::get<0>(r), rms_post_weight, gate_up_weight, down_weight, eps, split);
     return std::make_tuple(out, std::get<1>(r), std::get<2>(r));
 }
 
@@ -638,7 +643,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     });
     m.def("llama_decoder_layer_sglang", &llama_decoder_layer_sglang, py::arg("input"), py::arg("residual"), py::arg("weight_qkv"),
           py::arg("weight_o"), py::arg("k_cache"), py::arg("v_cache"), py::arg("rms_input_weight"), py::arg("eps"), py::arg("cos"),
-          py::arg("sin"), py::arg("num_heads") = 32);
+          py::arg("sin"), py::arg("num_heads") = 32, py::arg("split") = false);
     m.def("llama_decoder_layer", &llama_decoder_layer, py::arg("input"), py::arg("weight_qkv"), py::arg("weight_o"), py::arg("k_cache"),
           py::arg("v_cache"), py::arg("rms_input_weight"), py::arg("cos"), py::arg("sin"), py::arg("num_heads") = 32);
     m.def("llama_decoder_layer_batch_decode_sglang", &llama_decoder_layer_batch_decode_sglang, py::arg("output"),
@@ -646,21 +651,29 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("paged_kv_indptr"), py::arg("paged_kv_indices"), py::arg("k_cache_ptrs"), py::arg("v_cache_ptrs"),
           py::arg("layer_id"), py::arg("rms_input_weight"), py::arg("eps"), py::arg("positions"), py::arg("cos_sin"));
     m.def("llama_mlp", &llama_mlp, py::arg("input"), py::arg("rms_weight"), py::arg("gate_up_weight"), py::arg("down_weight"),
-          py::arg("eps"));
+          py::arg("eps"), py::arg("split") = false);
     m.def("llama_decoder_layer_full", &llama_decoder_layer_full, py::arg("input"), py::arg("weight_qkv"), py::arg("weight_o"),
           py::arg("k_cache"), py::arg("v_cache"), py::arg("rms_input_weight"), py::arg("rms_post_weight"),
           py::arg("gate_up_weight"), py::arg("down_weight"), py::arg("eps"), py::arg("cos"), py::arg("sin"),
-          py::arg("num_heads") = 32);
+          py::arg("num_heads") = 32, py::arg("split") = false);
     m.def("cfpp_version", []() { return std::string(cfpp_version()); });
     m.def("debug_set_trace", [](c10::optional<Tensor> buf) {
-        // int64 device tensor of at least 1024*16*16 elements, or None to switch tracing off
+        // profiling builds of the HIP library only (built with -DCFPP_TRACE): int64 device tensor of at least
+        // 1024*16*16 elements, or None to switch tracing off
+        typedef int (*set_trace_fn)(void*);
+        set_trace_fn fn = reinterpret_cast<set_trace_fn>(dlsym(RTLD_DEFAULT, "cfpp_debug_set_trace"));
+        TORCH_CHECK(fn != nullptr, "this build of libcfpp.so has no phase tracing (build it with CFPP_TRACE=1)");
         if (buf.has_value()) {
             TORCH_CHECK(buf->is_cuda() && buf->scalar_type() == torch::kInt64 && buf->is_contiguous() && buf->numel() >= 1024 * 16 * 16,
                         "trace buffer must be a contiguous int64 GPU tensor with >= 262144 elements");
-            cfpp_debug_set_trace(buf->data_ptr());
+            fn(buf->data_ptr());
         } else {
-            cfpp_debug_set_trace(nullptr);
+            fn(nullptr);
         }
+    });
+    m.def("device_status", [](bool clear) { return cfpp_device_status(clear ? 1 : 0); }, py::arg("clear") = false);
+    m.def("one_launch_fits", [](int64_t grid, int64_t cus, int64_t per_cu) {
+        return cfpp_one_launch_fits((int)grid, (int)cus, (int)per_cu) != 0;
     });
     m.def("workspace_bytes", [](int64_t hidden, int64_t heads, int64_t head_dim, int64_t rotary_dim, int64_t ffn) {
         cfpp_neox_dims d{(int32_t)hidden, (int32_t)heads, (int32_t)head_dim, (int32_t)rotary_dim, (int32_t)ffn, 1e-5f};
@@ -722,6 +735,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
             void* p = nullptr;
             check_rc(cfpp_stack_buffers(s.s, nullptr, &p, nullptr, nullptr, nullptr), "buffers");
             return torch::from_blob(p, {1, (int64_t)s.dims.hidden}, torch::TensorOptions().dtype(torch::kFloat16).device(s.device));
+        })
+        .def("check", [](PyStack& s) {
+            // synchronises; raises if a step of this stack raised a device-side failure flag
+            c10::hip::HIPGuardMasqueradingAsCUDA guard(s.device);
+            check_rc(cfpp_stack_check(s.s, cur_stream()), "NeoxStack.check");
         })
         .def("state", [](PyStack& s) {
             int32_t* p = nullptr;

@@ -107,7 +107,8 @@ class NeoxDecoder:
         self._stack.step()
 
     def graph_steps(self, n: int):
-        """`n` decode steps, each one replay of the captured hipGraph."""
+        """`n` decode steps, each one replay of the captured hipGraph.  Raises instead of stepping past the last
+        cache row."""
         self._stack.graph_steps(int(n))
 
     def profile_step(self):
@@ -127,6 +128,13 @@ class NeoxDecoder:
         """int32 `[token, seq_len, steps_done]` on the device."""
         return self._stack.state()
 
+    def check(self):
+        """Synchronises and raises RuntimeError if a step since the last check raised a device-side failure flag
+        (an expired bounded wait inside a fused launch, a position beyond the caches)."""
+        self._stack.check()
+
     def generated(self) -> List[int]:
+        """The tokens picked since `set_state`; raises if one of the steps failed on the device."""
+        self.check()
         n = int(self.state[2].item())
         return self._stack.history()[:n].tolist()

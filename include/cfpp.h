@@ -7,8 +7,17 @@
  *
  * Conventions for every call that returns `int`:
  *   0  success; <0 a `cfpp_status` argument error (nothing was launched); >0 a hipError_t.
- * No entry point throws or synchronises the device; only the ones whose comment says so
- * allocate device memory (context / stack creation).  All launches go to the given stream.
+ * No entry point throws or synchronises the device (the *_check calls excepted); only the ones whose
+ * comment says so allocate device memory (context / stack creation).  All launches go to the given stream.
+ *
+ * One-launch kernels and what they need.  CFPP_MODE_FUSED runs a whole layer as ONE launch whose workgroups wait
+ * for each other's results, so all of them must be on the device at the same time.  The library launches it only
+ * when the device can hold the whole grid (kernel occupancy x compute units, queried once per device and kernel)
+ * and takes the per-stage launches of CFPP_MODE_SPLIT otherwise: same results, bit for bit.  What it cannot see is
+ * other work on the device: while a fused launch runs, no other stream or process may keep compute units busy
+ * with long kernels.  Every wait inside the kernels is bounded (about a second); one that expires raises a failure
+ * flag instead of hanging, the results of that launch are invalid, and every later launching call on the device
+ * returns CFPP_ERR_DEVICE until cfpp_device_status(1) has been called (re-zero the workspaces that were in use).
  *
  * Tensor contract (same as the reference's dispatch code,
  * include/5090/pythia_2b8/pythia_kernel_dispatch.cu:4-75): fp16 row-major contiguous;
@@ -30,11 +39,13 @@ typedef enum cfpp_status {
     CFPP_OK = 0,
     CFPP_ERR_NULL = -1,        /* a required pointer is NULL */
     CFPP_ERR_DIMS = -2,        /* unsupported dimensions */
-    CFPP_ERR_SEQ = -3,         /* seq_len < 0 or seq_len > cache rows available */
+    CFPP_ERR_SEQ = -3,         /* seq_len < 0, beyond the cache rows, or (position-indexed RoPE tables) == cache rows */
     CFPP_ERR_WORKSPACE = -4,   /* workspace too small or misaligned */
     CFPP_ERR_CONTEXT = -5,     /* unknown / duplicate context id */
     CFPP_ERR_MODE = -6,        /* unknown mode */
-    CFPP_ERR_DEVICE = -7,      /* device-side failure flag raised (bounded wait expired, bad seq_len) */
+    CFPP_ERR_DEVICE = -7,      /* a device-side failure flag is raised (bounded wait expired, bad device seq_len):
+                                  by an earlier launch on this device (see cfpp_device_status) or in the workspace
+                                  that was checked */
     CFPP_ERR_ALIGN = -8,       /* a tensor pointer is not 16-byte aligned */
     CFPP_ERR_ALIAS = -9        /* an output overlaps an input it must not overlap */
 } cfpp_status;
@@ -133,6 +144,7 @@ typedef struct cfpp_llama_attn {
     const float* cos;        /* [>= D/2] fp32 */
     const float* sin;
     int32_t add_residual;    /* 0: output = W_o attn (the reference's op); 1: output = r + W_o attn (the layer's hidden state) */
+    int32_t mode;            /* cfpp_mode: one launch, or one launch per stage (same results) */
 } cfpp_llama_attn;
 
 size_t cfpp_llama_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim);
@@ -142,14 +154,16 @@ int cfpp_llama_attention_decode(const cfpp_llama_attn* a, void* workspace, size_
  * include/5090/llama/llama_kernel_dispatch.cu:4-145): output = W_o^T attn, no residual stream (residual must be NULL,
  * add_residual 0), weights stored [in, out]: w_qkv is [3H, H] = three [H_in, H_out] matrices for q, k, v stacked,
  * w_o is [H_in, H_out]; GPT-J pairing of the rotary dims (dim 2i with 2i+1; include/5090/llama/kernel.cuh:298-314)
- * with cos / sin tables of head_dim entries indexed by the dim (:280-281).  Caches are not written.
+ * with cos / sin tables of head_dim entries indexed by the dim (:280-281).  Caches are not written.  `mode` must be
+ * CFPP_MODE_FUSED (0): the op has one variant, three launches.
  * Workspace: cfpp_llama_plain_workspace_bytes, 256-byte aligned, zero-initialised once, one per stream. */
 size_t cfpp_llama_plain_workspace_bytes(int32_t hidden, int32_t heads, int32_t head_dim);
 int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- LLaMA MLP block ---------------------------------------------------------------------------------
  * output = input + W_down (silu(Wg n) * (Wu n)),  n = RMSNorm(input; eps) * rms_w,  w_gate_up = [Wg; Wu] ([2F, H]),
- * w_down [H, F].  One launch (norm, gated up rows in two phases, down rows + residual behind device-wide events).  The reference fuses only the
+ * w_down [H, F].  One launch (norm, gated up rows in two phases, down rows + residual behind device-wide events) or
+ * two (mode).  The reference fuses only the
  * attention block of a LLaMA layer (its test leaves the MLP commented out, reference tests/test_llama.py:108-110);
  * this completes the layer its benchmark configuration describes.
  * Workspace: cfpp_llama_mlp_workspace_bytes, 256-byte aligned, zero-initialised once, one per stream. */
@@ -161,6 +175,7 @@ typedef struct cfpp_llama_mlp_args {
     const void* w_down;      /* [H, F] fp16 */
     const void* input;       /* [H] fp16 */
     void* output;            /* [H] fp16 */
+    int32_t mode;            /* cfpp_mode: one launch, or two (gate/up rows, then down rows; same results) */
 } cfpp_llama_mlp_args;
 
 size_t cfpp_llama_mlp_workspace_bytes(int32_t hidden, int32_t ffn);
@@ -235,14 +250,24 @@ int cfpp_ctx_step(int family, int64_t id, const cfpp_neox_weights* w, const cfpp
 /* Frees the context's buffers; unknown id is a no-op returning CFPP_OK. */
 int cfpp_ctx_destroy(int family, int64_t id);
 
-/* Reads and clears the device-side failure flag of a workspace (synchronises `stream`).
- * Returns CFPP_OK or CFPP_ERR_DEVICE.  For tests and debugging; not on the hot path. */
+/* Reads and clears the device-side failure flag of a workspace (synchronises `stream`); a workspace with a raised
+ * flag is zeroed again.  Returns CFPP_OK or CFPP_ERR_DEVICE.  Not on the hot path.  cfpp_ctx_check / cfpp_stack_check
+ * (below) do the same for the workspace a context or a stack owns. */
 int cfpp_workspace_check(const cfpp_neox_dims* dims, void* workspace, void* stream);
+int cfpp_ctx_check(int family, int64_t id, void* stream);
 
-/* Debugging aid: when set to a device buffer of cfpp_debug_trace_bytes() bytes, every fused launch
- * stores 100 MHz timestamps of its phase boundaries per workgroup and wave
- * ([workgroup][16 waves][16 slots] int64); NULL switches it off.  No counterpart in the reference. */
-int cfpp_debug_set_trace(void* device_buffer);
+/* Failure flags raised by any launch on the current device since they were last cleared (bit 0: a bounded
+ * device-side wait expired; bit 1: a device-side seq_len was out of range), read from a word of pinned host memory
+ * that the kernels write on failure: no device synchronisation, callable at any time; flags of launches still
+ * running are seen once they got there.  `clear` != 0 resets the word.  While it is non-zero every launching entry
+ * point returns CFPP_ERR_DEVICE.  No counterpart in the reference (which checks no error at all). */
+int cfpp_device_status(int clear);
+
+/* The rule by which CFPP_MODE_FUSED decides whether a one-launch kernel may be launched: 1 when `grid` workgroups
+ * fit `compute_units` x `blocks_per_cu` resident workgroups, else 0 (the per-stage launches are taken).  The
+ * reference gets the same guarantee from cudaLaunchCooperativeKernel, which refuses a grid that cannot be
+ * co-resident (include/5090/pythia_2b8/pythia_kernel_dispatch.cu:242). */
+int cfpp_one_launch_fits(int grid, int compute_units, int blocks_per_cu);
 
 /* ---- whole-model greedy decode (our counterpart of the reference's Python decode loop,
  * tests/benchmark_decode.py:147-189: embedding row -> layers -> final LayerNorm -> LM head ->
@@ -268,7 +293,8 @@ typedef struct cfpp_neox_stack cfpp_neox_stack;   /* opaque */
 
 /* Allocates state (device int32 seq_len + token, hidden ping-pong, logits, workspace). */
 int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out);
-/* Sets the device-resident (token, seq_len) the next step starts from (async on `stream`). */
+/* Sets the device-resident (token, seq_len) the next step starts from (async on `stream`); seq_len < cache_rows.
+ * The step calls below return CFPP_ERR_SEQ instead of running past the last cache row. */
 int cfpp_stack_set_state(cfpp_neox_stack* s, int32_t token, int32_t seq_len, void* stream);
 /* One decode step launched eagerly: consumes (token, seq_len), appends K/V rows, writes logits,
  * then stores argmax as the new token and seq_len+1. */
@@ -283,6 +309,8 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
  * state int32[3] = {token, seq_len, steps done}, token history int32 [history_capacity]. */
 int cfpp_stack_buffers(cfpp_neox_stack* s, float** logits, void** hidden, int32_t** state,
                        int32_t** history, int32_t* history_capacity);
+/* cfpp_workspace_check for the stack's own workspace (synchronises `stream`). */
+int cfpp_stack_check(cfpp_neox_stack* s, void* stream);
 int cfpp_stack_destroy(cfpp_neox_stack* s);
 
 /* Final LayerNorm + LM-head GEMV: logits[v] = W[v,:] . LN(x) (no bias), fp32 logits.

@@ -476,3 +476,34 @@ def make_layer_inputs(dims: NeoxDims, seq_len: int, capacity: Optional[int] = No
     v[seq_len:] = 1e4
     cos, sin = rope_table(torch.tensor([seq_len]), dims.rotary_dim)
     return x.to(device), k.to(device), v.to(device), cos.to(device), sin.to(device)
+
+
+def make_reference_unit_test_inputs(dims: NeoxDims, seq_len: int = 129, seed: int = 42, zero_bias_o: bool = False,
+                                    pad_rope_to_head_dim: bool = False, ln_2d: bool = True):
+    """The inputs of the reference's own layer unit tests, drawn in their order from one CPU generator
+    (reference tests/test_pythia.py:15 seed 42, :162-164 every tensor `randn * 0.1` in fp16, :191-217 the order
+    input, weight_qkv, bias_qkv, weight_o, bias_o, the four LayerNorm tensors as `[1,H]`, the four MLP tensors, one
+    `[2, seqlen, H]` K/V block with exactly `seqlen` rows, :24-42 then RoPE from an independent uniform angle per
+    rotary entry, padded to `[1, D]` with cos 1 / sin 0; tests/test_pythia_6b9.py:47-51,196-228 is the same recipe
+    with a random bias_o and un-padded `[rot]` tables).  `zero_bias_o` / `pad_rope_to_head_dim` select the 2.8B
+    script's choices.  Returns (weights dict, x, k_cache, v_cache, cos, sin): the two halves of cos / sin do NOT repeat,
+    so a kernel that reads entry d mod rot/2 for dim d fails on these inputs."""
+    H, F, D, rot = dims.hidden, dims.ffn, dims.head_dim, dims.rotary_dim
+    g = torch.Generator().manual_seed(seed)
+    rn = lambda *shape: (torch.randn(shape, generator=g) * 0.1).half()
+    x = rn(1, H)
+    w = {"w_qkv": rn(3 * H, H), "b_qkv": rn(3 * H), "w_o": rn(H, H)}
+    w["b_o"] = torch.zeros(H, dtype=torch.float16) if zero_bias_o else rn(H)
+    for name in ("ln_w", "ln_b", "post_ln_w", "post_ln_b"):
+        t = rn(1, H)
+        w[name] = t if ln_2d else t.reshape(H)
+    w["w_up"], w["b_up"], w["w_down"], w["b_down"] = rn(F, H), rn(F), rn(H, F), rn(H)
+    kv = rn(2, seq_len, H)
+    ang = torch.rand((1, rot), generator=g, dtype=torch.float32) * (2 * math.pi)
+    cos, sin = torch.cos(ang), torch.sin(ang)
+    if pad_rope_to_head_dim:
+        cos = torch.cat([cos, torch.ones((1, D - rot))], dim=-1)
+        sin = torch.cat([sin, torch.zeros((1, D - rot))], dim=-1)
+    else:
+        cos, sin = cos.reshape(rot), sin.reshape(rot)
+    return w, x, kv[0].contiguous(), kv[1].contiguous(), cos.contiguous(), sin.contiguous()

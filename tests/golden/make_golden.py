@@ -61,12 +61,32 @@ def llama_batch_inputs(name):
     return (dims, layer_id) + tuple(O.make_llama_batch_inputs(dims, lens, seed=seed, w_std=0.05))
 
 
+# The reference's own unit-test inputs (oracle.make_reference_unit_test_inputs: reference tests/test_pythia.py:15,24-42,
+# 162-230 and the 6.9B twin): dims, zero bias_o, RoPE tables padded to [1, D]
+REFERENCE_RECIPE_CASES = {
+    "pythia_2b8_reference_recipe_s129": (O.PYTHIA_2B8, True, True),
+    "pythia_6b9_reference_recipe_s129": (O.PYTHIA_6B9, False, False),
+}
+
+
+def reference_recipe_inputs(name):
+    dims, zero_bo, pad = REFERENCE_RECIPE_CASES[name]
+    return (dims,) + tuple(O.make_reference_unit_test_inputs(dims, 129, zero_bias_o=zero_bo, pad_rope_to_head_dim=pad))
+
+
 def new_rows(indptr, indices):
     return [int(indices[int(indptr[b + 1]) - 1]) for b in range(indptr.numel() - 1)]
 
 
 def main():
     torch.set_num_threads(max(1, os.cpu_count() or 1))
+    for name in REFERENCE_RECIPE_CASES:
+        dims, w, x, k, v, cos, sin = reference_recipe_inputs(name)
+        r = O.neox_layer_decode(x, w, k, v, cos, sin, 129, dims, dtype=torch.float64, round_io=True)
+        out = {n: r[n].to(torch.float32).numpy() for n in ("output", "k_new", "v_new")}
+        path = os.path.join(HERE, name + ".npz")
+        np.savez_compressed(path, **out)
+        print(name, {n: a.shape for n, a in out.items()}, os.path.getsize(path), "bytes")
     for name in LLAMA_PLAIN_CASES:
         dims, w, x, k, v, cos, sin = llama_plain_inputs(name)
         r = O.llama_attention_plain(x, w, k, v, cos, sin, dims, dtype=torch.float64, round_io=True)

@@ -76,6 +76,50 @@ def test_null_and_mode_errors_launch_nothing(lib):
     assert lib.cfpp_neox_lm_head(4096, 100, ctypes.c_float(1e-5), None, None, None, None, None, None) == -1
 
 
+def test_one_launch_rule_and_device_status_without_a_gpu(lib):
+    """The routing rule of the fused mode: a grid is launched in one piece only if it fits compute units x occupancy."""
+    fits = lib.cfpp_one_launch_fits
+    assert fits(256, 256, 1) == 1 and fits(256, 256, 2) == 1 and fits(512, 256, 2) == 1
+    assert fits(257, 256, 1) == 0 and fits(256, 128, 1) == 0 and fits(256, 255, 1) == 0
+    assert fits(256, 256, 0) == 0            # the kernel does not fit a compute unit at all (or the query failed)
+    assert fits(0, 256, 1) == 0 and fits(256, 0, 1) == 0 and fits(-1, 256, 1) == 0
+    assert fits(1 << 30, 1 << 30, 4) == 1    # no overflow in the product
+    assert lib.cfpp_device_status(0) == 0 and lib.cfpp_device_status(1) == 0
+    assert lib.cfpp_ctx_check(0, ctypes.c_int64(4242), None) == -5          # unknown context
+    assert lib.cfpp_stack_check(None, None) == -1
+
+
+class NeoxIo(ctypes.Structure):
+    _fields_ = [("input", ctypes.c_void_p), ("output", ctypes.c_void_p), ("k_new", ctypes.c_void_p), ("v_new", ctypes.c_void_p),
+                ("k_cache", ctypes.c_void_p), ("v_cache", ctypes.c_void_p), ("cache_rows", ctypes.c_int32),
+                ("cos", ctypes.c_void_p), ("sin", ctypes.c_void_p), ("rope_stride", ctypes.c_int32), ("seq_len", ctypes.c_int32),
+                ("d_seq_len", ctypes.c_void_p), ("max_seq_len", ctypes.c_int32), ("attn_output", ctypes.c_void_p),
+                ("mlp_intermediate", ctypes.c_void_p)]
+
+
+def test_sequence_length_rules_are_checked_before_any_launch(lib):
+    """seq_len may equal the cache rows only when the append can be skipped and cos / sin are the position's own row;
+    with position-indexed tables or a device-side length the position needs a row of its own."""
+    d = Dims(2560, 32, 80, 20, 10240, 1e-5)
+    w = (ctypes.c_void_p * 12)(*([4096] * 12))
+    lib.cfpp_neox_workspace_bytes.restype = ctypes.c_size_t
+    n = lib.cfpp_neox_workspace_bytes(ctypes.byref(d))
+    ws = ctypes.c_void_p(1 << 20)
+
+    def call(**kw):
+        io = NeoxIo(input=4096, output=4096, k_new=4096, v_new=4096, k_cache=4096, v_cache=4096, cache_rows=10, cos=4096, sin=4096,
+                    rope_stride=0, seq_len=0, d_seq_len=None, max_seq_len=0, attn_output=None, mlp_intermediate=None)
+        for k, v in kw.items():
+            setattr(io, k, v)
+        return lib.cfpp_neox_layer_decode(ctypes.byref(d), w, ctypes.byref(io), 7 if kw.get("_mode") else 0, ws, ctypes.c_size_t(n), None)
+
+    assert call(seq_len=11) == -3 and call(seq_len=-1) == -3 and call(cache_rows=-1) == -3
+    assert call(seq_len=10, rope_stride=20) == -3            # the table has no row for position 10
+    assert call(seq_len=3, rope_stride=-20) == -3
+    assert call(d_seq_len=4096, cache_rows=0) == -3          # a device-side length always appends
+    assert call(seq_len=3, cos=4100) == -8                   # misaligned pointer: still an argument error, nothing launched
+
+
 class LlamaBatch(ctypes.Structure):
     _fields_ = [("hidden", ctypes.c_int32), ("heads", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("eps", ctypes.c_float),
                 ("batch", ctypes.c_int32), ("layer_id", ctypes.c_int32)] + [(n, ctypes.c_void_p) for n in (

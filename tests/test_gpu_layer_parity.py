@@ -21,13 +21,13 @@ def _cos(a, b):
     return float((a @ b) / (a.norm() * b.norm() + 1e-30))
 
 
-def assert_close(name, got, want):
+def assert_close(name, got, want, max_abs=MAX_ABS):
     got, want = got.detach().cpu().float(), want.detach().cpu().float()
     assert got.shape == want.shape, (name, got.shape, want.shape)
     err = float((got - want).abs().max())
     cs = _cos(got, want)
     print(f"  {name}: max-abs {err:.3e} cosine {cs:.7f}", flush=True)
-    assert err <= MAX_ABS, f"{name}: max-abs {err} > {MAX_ABS}"
+    assert err <= max_abs, f"{name}: max-abs {err} > {max_abs}"
     assert cs >= MIN_COS, f"{name}: cosine {cs} < {MIN_COS}"
 
 

@@ -16,14 +16,14 @@ def cf():
     return clusterfusion
 
 
-def run(cf, dims, S, seed, w_std=0.02):
+def run(cf, dims, S, seed, w_std=0.02, split=False):
     w, x, res, k, v, cos, sin = O.make_llama_attn_inputs(dims, S, seed=seed, w_std=w_std)
     ref = O.llama_attention_sglang(x, res, w, k, v, cos, sin, dims)
     dev = "cuda:0"
     res_g = res.to(dev)
     kg, vg = k.to(dev), v.to(dev)
     out, res_out, kn, vn = cf.llama_decoder_layer_sglang(x.to(dev), res_g, w["w_qkv"].to(dev), w["w_o"].to(dev), kg, vg,
-                                                         w["rms1"].to(dev), dims.eps, cos.to(dev), sin.to(dev), dims.heads)
+                                                         w["rms1"].to(dev), dims.eps, cos.to(dev), sin.to(dev), dims.heads, split)
     torch.cuda.synchronize()
     return ref, out, res_out, res_g, kn, vn, (k, v, kg, vg)
 
@@ -52,6 +52,27 @@ def test_small_geometry_and_determinism(cf):
     assert_close("k_new", kn, ref["k_new"])
     _, out2, _, _, kn2, _, _ = run(cf, dims, 333, seed=5, w_std=0.05)
     assert torch.equal(out, out2) and torch.equal(kn, kn2)
+
+
+@pytest.mark.parametrize("S", [1024, 0])
+def test_one_launch_per_stage_gives_the_same_bits(cf, S):
+    """mode = split (QKV rows, attention items, O rows as three launches; gate/up rows and down rows as two): what the
+    library falls back to when a device cannot hold a one-launch grid.  Same results, bit for bit."""
+    print(f"\ncase llama2-7b split launches S={S}", flush=True)
+    dims = O.LLAMA2_7B
+    ref, out, _, res_g, kn, vn, _ = run(cf, dims, S, seed=70 + S)
+    _, out_s, _, res_s, kn_s, vn_s, _ = run(cf, dims, S, seed=70 + S, split=True)
+    assert torch.equal(out, out_s) and torch.equal(kn, kn_s) and torch.equal(vn, vn_s) and torch.equal(res_g, res_s)
+    assert_close("output", out_s, ref["output"])
+    w = _full_layer_weights(dims, seed=6)
+    g = torch.Generator().manual_seed(32)
+    h = torch.randn(1, dims.hidden, generator=g).half()
+    dev = "cuda:0"
+    a = [h.to(dev), w["rms2"].to(dev), w["w_gate_up"].to(dev), w["w_down"].to(dev), dims.eps]
+    one, two = cf.llama_mlp(*a), cf.llama_mlp(*a, split=True)
+    torch.cuda.synchronize()
+    assert torch.equal(one, two)
+    assert_close("mlp output", two, O.llama_mlp(h, w, dims)["output"])
 
 
 def test_argument_errors(cf):

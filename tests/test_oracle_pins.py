@@ -359,3 +359,61 @@ def test_llama_attention_plain_is_the_sglang_block_with_transposed_weights_and_g
     # S = 0: the only key is the new token
     r0 = O.llama_attention_plain(x, wt, k[:0], v[:0], c2, s2, dims, dtype=torch.float64, round_io=False)
     assert torch.allclose(r0["attn_heads"], r0["v_new"][0], atol=1e-12, rtol=0)
+
+
+# ---------------------------------------------------------------- the reference's own unit-test inputs
+# (tests/test_pythia.py:24-42: an independent angle per rotary entry, so entries d and d + rot/2 of cos / sin differ)
+@pytest.mark.parametrize("dims,zero_bo,pad", [(TINY, True, True), (NeoxDims(320, 4, 80, 20, 1280), True, True),
+                                              (SMALL, False, False)])
+def test_reference_recipe_inputs_against_hf_layer_and_brute_force(dims, zero_bo, pad):
+    from oracle import hf_neox
+    S = 7
+    w, x, k, v, cos, sin = O.make_reference_unit_test_inputs(dims, seq_len=S, zero_bias_o=zero_bo, pad_rope_to_head_dim=pad)
+    rot = dims.rotary_dim
+    assert cos.numel() == (dims.head_dim if pad else rot) and k.shape == (S, dims.hidden)
+    assert not torch.allclose(cos.reshape(-1)[: rot // 2], cos.reshape(-1)[rot // 2: rot])      # the halves do not repeat
+    if pad:
+        assert torch.equal(cos.reshape(-1)[rot:], torch.ones(dims.head_dim - rot)) and float(sin.reshape(-1)[rot:].abs().max()) == 0.0
+    assert (float(w["b_o"].abs().max()) == 0.0) == zero_bo and w["ln_w"].shape == (1, dims.hidden)
+    r = O.neox_layer_decode(x, w, k, v, cos, sin, S, dims, dtype=torch.float64, round_io=False)
+    wf = {n: t.reshape(-1) if n.startswith(("ln_", "post_ln_")) else t for n, t in w.items()}
+    layer = hf_neox.build_hf_layer(dims, wf, dtype=torch.float64)
+    out, k_new, v_new = hf_neox.hf_layer_decode(layer, x, k, v, cos, sin, S, dims, dtype=torch.float64)
+    assert torch.allclose(r["output"], out, atol=1e-6, rtol=0)
+    assert torch.allclose(r["k_new"], k_new, atol=1e-12, rtol=0) and torch.allclose(r["v_new"], v_new, atol=1e-12, rtol=0)
+    if dims.hidden <= 64:
+        bo, bk, bv = _brute_force_layer(x, wf, k, v, cos, sin, S, dims)
+        assert torch.allclose(r["output"].reshape(-1), torch.tensor(bo, dtype=torch.float64), atol=1e-10)
+        assert torch.allclose(r["k_new"].reshape(-1), torch.tensor(bk, dtype=torch.float64).reshape(-1), atol=1e-12)
+    # a table whose second half is overwritten with the first gives a different rotation: the two conventions are
+    # told apart by these inputs
+    c2 = cos.clone().reshape(-1); c2[rot // 2: rot] = c2[: rot // 2]
+    s2 = sin.clone().reshape(-1); s2[rot // 2: rot] = s2[: rot // 2]
+    other = O.neox_layer_decode(x, w, k, v, c2, s2, S, dims, dtype=torch.float64, round_io=False)
+    assert float((other["k_new"] - r["k_new"]).abs().max()) > 1e-3
+
+
+def test_llama_attention_plain_rotates_q_as_well():
+    """q of the plain op under non-zero angles: the attention output must be that of the GPT-J-rotated q against the
+    returned (rotated) keys; an unrotated q gives a different result."""
+    dims, S, w, x, res, k, v, cos, sin = _tiny_llama()
+    H, D, nh = dims.hidden, dims.head_dim, dims.heads
+    wt = {"rms1": w["rms1"], "w_qkv_t": w["w_qkv"].reshape(3, H, H).transpose(1, 2).contiguous().reshape(3 * H, H),
+          "w_o_t": w["w_o"].t().contiguous()}
+    g = torch.Generator().manual_seed(10)
+    ang = torch.rand(D // 2, generator=g, dtype=torch.float64) * 6.28
+    c2, s2 = torch.repeat_interleave(torch.cos(ang), 2), torch.repeat_interleave(torch.sin(ang), 2)
+    r = O.llama_attention_plain(x, wt, k, v, c2, s2, dims, dtype=torch.float64, round_io=False)
+    n1 = O.rms_norm(x.double().reshape(1, H), w["rms1"].double(), 1e-6)
+    q_raw = (n1 @ wt["w_qkv_t"].double().reshape(3, H, H)[0]).reshape(nh, D)
+    keys = torch.cat([k.double().reshape(S, nh, D), r["k_new"]], dim=0).permute(1, 0, 2)
+    vals = torch.cat([v.double().reshape(S, nh, D), r["v_new"]], dim=0).permute(1, 0, 2)
+
+    def heads(q):
+        p = torch.softmax(torch.einsum("hd,hsd->hs", q, keys) / math.sqrt(D), dim=-1)
+        return torch.einsum("hs,hsd->hd", p, vals)
+    # HF's GPT-J rotation of q (third party), as test_rope_pairs_gptj_matches_hf_gptj_rotary uses it
+    from transformers.models.gptj.modeling_gptj import apply_rotary_pos_emb as gptj_rope
+    q_rot = gptj_rope(q_raw[None, None], s2[None, None, 0::2], c2[None, None, 0::2])[0, 0]
+    assert torch.allclose(r["attn_heads"], heads(q_rot), atol=1e-12, rtol=0)
+    assert float((r["attn_heads"] - heads(q_raw)).abs().max()) > 1e-4
