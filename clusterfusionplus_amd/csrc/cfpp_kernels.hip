@@ -1141,6 +1141,17 @@ struct DeviceInfo {
 };
 std::mutex g_device_mu;
 
+// Scratch memory of cfpp_neox_layer_decode_static, the entry point that allocates nothing: one array per device,
+// part of the library's code object, held by every device the library runs on until the process ends.  Host code
+// must not use the array's name as an address (on the host it is a stand-in, not device memory): the address of
+// a device's copy comes from hipGetSymbolAddress, once per device (static_scratch_address).
+constexpr size_t kStaticScratchBytes = 1280u << 10;      // 1.25 MiB: a Pythia-6.9B layer needs 1.19 MiB
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// set while an entry point that must not allocate runs on this thread: the per-device set-up then skips the pinned
+// status word (it is added by the next ordinary call)
+thread_local bool tl_no_alloc = false;
+
 DeviceInfo& device_info() {
     static DeviceInfo info[64];
     int dev = 0;
@@ -1152,23 +1163,47 @@ DeviceInfo& device_info() {
             hipDeviceProp_t prop;
             if (hipGetDeviceProperties(&prop, dev) == hipSuccess) {
                 d.cus = prop.multiProcessorCount;
-                void* h = nullptr;
-                if (hipHostMalloc(&h, 64, hipHostMallocMapped) == hipSuccess && h != nullptr) {
-                    *reinterpret_cast<volatile int*>(h) = 0;
-                    void* dp = nullptr;
-                    if (hipHostGetDevicePointer(&dp, h, 0) == hipSuccess && dp != nullptr) {
-                        d.host_status = reinterpret_cast<int*>(h);
-                        d.host_status_dev = reinterpret_cast<int*>(dp);
-                    } else {
-                        (void)hipHostFree(h);
-                    }
-                }
-                (void)hipGetLastError();
                 d.ok = true;
             }
+            (void)hipGetLastError();
+        }
+    }
+    if (d.ok && d.host_status == nullptr && !tl_no_alloc) {
+        std::lock_guard<std::mutex> lock(g_device_mu);
+        if (d.host_status == nullptr) {
+            void* h = nullptr;
+            if (hipHostMalloc(&h, 64, hipHostMallocMapped) == hipSuccess && h != nullptr) {
+                *reinterpret_cast<volatile int*>(h) = 0;
+                void* dp = nullptr;
+                if (hipHostGetDevicePointer(&dp, h, 0) == hipSuccess && dp != nullptr) {
+                    d.host_status_dev = reinterpret_cast<int*>(dp);
+                    d.host_status = reinterpret_cast<int*>(h);
+                } else {
+                    (void)hipHostFree(h);
+                }
+            }
+            (void)hipGetLastError();
         }
     }
     return d;
+}
+
+// The address of the current device's copy of `scratch`, looked up on first use per device.
+int static_scratch_address(void** out) {
+    DeviceInfo& di = device_info();
+    if (!di.ok) return (int)hipErrorNoDevice;
+    if (di.static_scratch == nullptr) {
+        std::lock_guard<std::mutex> lock(g_device_mu);
+        if (di.static_scratch == nullptr) {
+            void* ptr = nullptr;
+            const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) return (int)e;
+            if (ptr == nullptr || (reinterpret_cast<uintptr_t>(ptr) & 255u)) return (int)hipErrorInvalidSymbol;
+            di.static_scratch = ptr;
+        }
+    }
+    *out = di.static_scratch;
+    return CFPP_OK;
 }
 
 // non-zero: some launch on this device has raised a failure flag since the word was last cleared
@@ -1598,6 +1633,7 @@ const char* cfpp_status_str(int s) {
         case CFPP_ERR_DEVICE: return "device-side failure flag raised";
         case CFPP_ERR_ALIGN: return "tensor pointer is not 16-byte aligned";
         case CFPP_ERR_ALIAS: return "an output overlaps an input";
+        case CFPP_ERR_STATIC_SCRATCH: return "the layer needs more scratch than the static array of the allocation-free entry point holds";
         default: break;
     }
     if (s > 0) return hipGetErrorString((hipError_t)s);
@@ -1618,6 +1654,40 @@ int cfpp_neox_layer_decode(const cfpp_neox_dims* dims, const cfpp_neox_weights* 
     if (rc) return rc;
     CFPP_REFUSE_AFTER_FAILURE();
     return run_layer(pl, p, mode, seq_hint_of(io), reinterpret_cast<hipStream_t>(stream));
+}
+
+int cfpp_init(void) {
+    DeviceInfo& di = device_info();          // compute units, pinned status word
+    if (!di.ok) return (int)hipErrorNoDevice;
+    void* ptr = nullptr;
+    return static_scratch_address(&ptr);     // this device's copy of the static scratch array
+}
+
+size_t cfpp_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int cfpp_neox_layer_decode_static(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io, int mode,
+                                  void* stream) {
+    if (mode != CFPP_MODE_FUSED && mode != CFPP_MODE_SPLIT) return CFPP_ERR_MODE;
+    int rc = check_dims(dims);
+    if (rc) return rc;
+    const WorkspaceLayout L = workspace_layout(*dims);
+    if (L.total > kStaticScratchBytes) return CFPP_ERR_STATIC_SCRATCH;
+    struct NoAlloc { NoAlloc() { tl_no_alloc = true; } ~NoAlloc() { tl_no_alloc = false; } } guard;
+    void* ws = nullptr;
+    if ((rc = static_scratch_address(&ws))) return rc;
+    LayerParams p;
+    Plan pl;
+    if ((rc = fill_params(dims, w, io, ws, kStaticScratchBytes, true, true, &p, &pl))) return rc;
+    CFPP_REFUSE_AFTER_FAILURE();
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    // The array keeps what the last call left there, possibly under another geometry's layout: the words that must
+    // start at zero (arrival counters, event counters, mailboxes, ticket counters, launch generation) are cleared by
+    // a small kernel in front of the layer (not a memset node: the call may be recorded into a graph).
+    const size_t words = (L.total - L.head_cnt) / 4;
+    hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, st,
+                       reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + L.head_cnt), words);
+    if ((rc = launch_check())) return rc;
+    return run_layer(pl, p, mode, seq_hint_of(io), st);
 }
 
 int cfpp_neox_attention_mlp_up(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io,

@@ -47,7 +47,8 @@ typedef enum cfpp_status {
                                   by an earlier launch on this device (see cfpp_device_status) or in the workspace
                                   that was checked */
     CFPP_ERR_ALIGN = -8,       /* a tensor pointer is not 16-byte aligned */
-    CFPP_ERR_ALIAS = -9        /* an output overlaps an input it must not overlap */
+    CFPP_ERR_ALIAS = -9,       /* an output overlaps an input it must not overlap */
+    CFPP_ERR_STATIC_SCRATCH = -10  /* cfpp_neox_layer_decode_static: the geometry needs more than cfpp_static_scratch_bytes() */
 } cfpp_status;
 
 /* Layer geometry.  Pythia-2.8B = {2560,32,80,20,10240,1e-5}, Pythia-6.9B = {4096,32,128,32,16384,1e-5}
@@ -109,6 +110,24 @@ size_t cfpp_neox_workspace_bytes(const cfpp_neox_dims* dims);
  * pythia_kernel_dispatch_split.cu:18-218) in CFPP_MODE_SPLIT. */
 int cfpp_neox_layer_decode(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io,
                            int mode, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same layer step for callers that cannot allocate device memory or pass a workspace around: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * The scratch memory that cfpp_neox_layer_decode takes as `workspace` is here an array inside the library
+ * (cfpp_static_scratch_bytes() = 1.25 MiB per device, held until the process ends); the call allocates nothing and
+ * frees nothing.  Geometries whose cfpp_neox_workspace_bytes exceeds that size return CFPP_ERR_STATIC_SCRATCH (both
+ * Pythia models fit).  All calls on one device share the one array: calls on the same stream are ordered and fine,
+ * calls that overlap in time on one device (two streams, two threads) race and give wrong results.  Every call
+ * first clears the array's counters and flags with a small kernel (it keeps the previous call's contents), then
+ * runs the same kernels as cfpp_neox_layer_decode: identical results, bit for bit.  The first call on a device looks
+ * up the device's copy of the array; call cfpp_init() beforehand (device current) when that first call may sit
+ * inside a graph capture. */
+int cfpp_neox_layer_decode_static(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io,
+                                  int mode, void* stream);
+size_t cfpp_static_scratch_bytes(void);
+/* Per-device set-up for the current device, done lazily by the other calls otherwise: compute-unit count, the
+ * pinned failure-flag word (the one allocation, host memory), the address of the static scratch array. */
+int cfpp_init(void);
 
 /* First half of the split API: LN, QKV, RoPE, append, attention, O-proj (+b_o) -> io->attn_output,
  * and MLP-up + GELU -> io->mlp_intermediate; k_new / v_new / cache row as in the full layer.

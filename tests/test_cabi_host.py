@@ -41,8 +41,8 @@ def test_status_strings_and_version(lib):
     lib.cfpp_status_str.restype = ctypes.c_char_p
     lib.cfpp_version.restype = ctypes.c_char_p
     assert lib.cfpp_status_str(0) == b"ok"
-    seen = {lib.cfpp_status_str(-i) for i in range(1, 10)}
-    assert len(seen) == 9 and b"unknown status" not in seen
+    seen = {lib.cfpp_status_str(-i) for i in range(1, 11)}
+    assert len(seen) == 10 and b"unknown status" not in seen
     assert b"gfx950" in lib.cfpp_version()
 
 
@@ -118,6 +118,26 @@ def test_sequence_length_rules_are_checked_before_any_launch(lib):
     assert call(seq_len=3, rope_stride=-20) == -3
     assert call(d_seq_len=4096, cache_rows=0) == -3          # a device-side length always appends
     assert call(seq_len=3, cos=4100) == -8                   # misaligned pointer: still an argument error, nothing launched
+
+
+def test_static_entry_point_argument_errors_launch_nothing(lib):
+    """The allocation-free layer step: bad mode, bad geometry and a geometry beyond its built-in scratch array are
+    refused before any HIP call."""
+    lib.cfpp_static_scratch_bytes.restype = ctypes.c_size_t
+    lib.cfpp_neox_workspace_bytes.restype = ctypes.c_size_t
+    cap = lib.cfpp_static_scratch_bytes()
+    assert cap == 1280 * 1024
+    for d in (Dims(2560, 32, 80, 20, 10240, 1e-5), Dims(4096, 32, 128, 32, 16384, 1e-5)):
+        assert lib.cfpp_neox_workspace_bytes(ctypes.byref(d)) <= cap
+    d = Dims(4096, 32, 128, 32, 16384, 1e-5)
+    assert lib.cfpp_neox_layer_decode_static(ctypes.byref(d), None, None, 5, None) == -6
+    assert lib.cfpp_neox_layer_decode_static(None, None, None, 0, None) == -1
+    assert lib.cfpp_neox_layer_decode_static(ctypes.byref(Dims(4096, 32, 128, 33, 16384, 1e-5)), None, None, 0, None) == -2
+    wide = Dims(4096, 512, 8, 8, 16384, 1e-5)
+    assert lib.cfpp_neox_workspace_bytes(ctypes.byref(wide)) > cap
+    assert lib.cfpp_neox_layer_decode_static(ctypes.byref(wide), None, None, 0, None) == -10
+    lib.cfpp_status_str.restype = ctypes.c_char_p
+    assert b"static" in lib.cfpp_status_str(-10)
 
 
 class LlamaBatch(ctypes.Structure):
