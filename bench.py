@@ -22,10 +22,23 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch of the fused layer kernel (fetched + written) from the committed hardware-counter
-# summary (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the 256 MiB calibration copy), keyed by
-# (model, context); other workloads have no counter run and report null.
-MEASURED_TRAFFIC_BYTES = {("pythia_6b9", 2048): 439.3e6 + 2.29e6}
+
+
+def recorded_traffic(model, ctx):
+    """HBM bytes per launch of the fused layer kernel (fetched + written) as recorded in the committed hardware-counter
+    summary of this workload (two `rocprofv3 --pmc` runs of this script, FETCH_SIZE and WRITE_SIZE, scaled by the
+    256 MiB calibration copy): the number on the summary's `traffic_bytes_per_launch:` line and the file it came from,
+    or (None, None) when no summary exists for the workload.  A counter run cannot be part of a timed run; the
+    summary states the command and the commit it was taken at."""
+    rel = os.path.join("profiles", f"k_fused_{model}_ctx{ctx}_hbm_traffic.txt")
+    try:
+        with open(os.path.join(ROOT, rel)) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1].split()[0]), rel
+    except OSError:
+        pass
+    return None, None
 
 
 def log(*a):
@@ -71,7 +84,100 @@ def build_model(cfg, rows, ctx, device, mode):
     k_caches = [rn((rows, H), 1.0) for _ in range(cfg.n_layers)]
     v_caches = [rn((rows, H), 1.0) for _ in range(cfg.n_layers)]
     dec = pkg.NeoxDecoder(cfg, layers, embed, fw, fb, lm_head, k_caches, v_caches, mode=mode)
+    dec.tensors = dict(layers=layers, embed=embed, final_ln_w=fw, final_ln_b=fb, lm_head=lm_head, k_caches=k_caches, v_caches=v_caches)
     return dec
+
+
+def time_tokens(dec, stream, ctx, tokens, warm):
+    """TPOT in ms of `tokens` graph replays starting at context `ctx` + `warm`, HIP events on the launch stream."""
+    import torch
+    dec.set_state(11, ctx)
+    dec.graph_steps(warm)
+    stream.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    dec.graph_steps(tokens)
+    e1.record(stream)
+    stream.synchronize()
+    return e0.elapsed_time(e1) / tokens
+
+
+def context_sweep(dec, cfg, stream, contexts, tokens=24, warm=4):
+    """TPOT and fraction of the 8 TB/s roofline at several contexts, on the model that is already resident."""
+    out = []
+    for c in contexts:
+        tpot = time_tokens(dec, stream, c, tokens, warm)
+        sb = step_bytes(cfg, c + warm + tokens // 2)
+        out.append({"context": c, "tokens": tokens, "tpot_ms": round(tpot, 4), "bytes": sb,
+                    "hbm_gbps": round(sb / (tpot * 1e-3) / 1e9, 1), "frac_of_peak": round(sb / (tpot * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+        log(f"[sweep] context {c}: {tpot:.4f} ms/token = {out[-1]['frac_of_peak'] * 100:.1f} % of peak")
+    dec.check()
+    return out
+
+
+def drop_in_loop(model, cfg, dec, ctx, tokens=24, warm=4):
+    """The reference's own per-token flow through the drop-in ops (reference tests/benchmark_decode.py:225-284): one
+    context per layer, per token the embedding row, 32 x `<model>_graph_decode_step`, `F.layer_norm`, the LM head
+    matmul and argmax in torch.  The reference runs that Python loop eagerly; here the position lives in a device int32
+    (the step op accepts one), so the loop is captured once with torch.cuda.graph and replayed per token."""
+    import torch
+    import clusterfusion as cf
+    t = dec.tensors
+    L, H, dev = cfg.n_layers, cfg.hidden, t["embed"].device
+    create, step, destroy = (getattr(cf, f"{model}_{n}") for n in ("create_graph_context", "graph_decode_step", "destroy_graph_context"))
+    rows = t["k_caches"][0].shape[0]
+    base = 1000
+    for l, w in enumerate(t["layers"]):
+        create(base + l, t["k_caches"][l], t["v_caches"][l], w["w_qkv"], w["w_o"], w["w_up"], w["w_down"], rows)
+    seq = torch.tensor([ctx], dtype=torch.int32, device=dev)
+    tok = torch.tensor([11], dtype=torch.int64, device=dev)
+
+    def one_token():
+        h = t["embed"].index_select(0, tok)
+        for l, w in enumerate(t["layers"]):
+            h, _, _ = step(base + l, h, w["ln_w"], w["ln_b"], w["b_qkv"], w["b_o"], dec.cos, dec.sin, t["k_caches"][l], t["v_caches"][l],
+                           w["post_ln_w"], w["post_ln_b"], w["b_up"], w["b_down"], seq)
+        h = torch.nn.functional.layer_norm(h, (H,), t["final_ln_w"], t["final_ln_b"], eps=cfg.eps)
+        logits = torch.matmul(h, t["lm_head"].t())
+        tok.copy_(torch.argmax(logits, dim=-1))
+        seq.add_(1)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        one_token()                      # warm-up outside the capture (library handles, lazy initialisation)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(4):
+        one_token()                      # the reference's way: the Python loop, launched eagerly
+    e1.record()
+    torch.cuda.synchronize()
+    eager = e0.elapsed_time(e1) / 4
+    eager_wall = (time.perf_counter() - t0) * 1e3 / 4
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        one_token()
+    seq.fill_(ctx)
+    for _ in range(warm):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(tokens):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    tpot = e0.elapsed_time(e1) / tokens
+    assert int(seq.item()) == ctx + warm + tokens
+    for l in range(L):
+        destroy(base + l)                # raises if a step of the context failed on the device
+    sb = step_bytes(cfg, ctx + warm + tokens // 2)
+    return {"workload": f"{model}: per-layer contexts, {L} x {model}_graph_decode_step per token with a device current_seq_len, final "
+                        "LayerNorm + LM head + argmax in torch, captured once with torch.cuda.graph and replayed",
+            "context": ctx, "tokens": tokens, "tpot_ms": round(tpot, 4), "frac_of_peak": round(sb / (tpot * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "eager_python_loop_tpot_ms": round(max(eager, eager_wall), 4)}
 
 
 def cpu_baseline(cfg, S, budget_s=12.0):
@@ -257,22 +363,22 @@ def other_workloads(pkg, dev, args):
 
     def stack_2b8():
         cfg, ctx, K, W = pkg.PYTHIA_2B8, 1024, 64, 8
-        dec = build_model(cfg, ctx + W + K + 40, ctx, dev, "fused")
+        dec = build_model(cfg, 4096 + 64, ctx, dev, "fused")
         stream = torch.cuda.Stream()
         with torch.cuda.stream(stream):
             dec.set_state(11, ctx)
-            dec.graph_steps(W)
-            stream.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            dec.graph_steps(K)
-            e1.record(stream)
-            stream.synchronize()
-        tpot = e0.elapsed_time(e1) / K
+            per_layer, _lm, _total = dec.profile_step()
+            tpot = time_tokens(dec, stream, ctx, K, W)
+            sweep = context_sweep(dec, cfg, stream, [2048, 4096])
         sb = step_bytes(cfg, ctx + W + K // 2)
+        lay_us = sorted(per_layer)[len(per_layer) // 2] * 1e3
+        first = {"context": ctx, "tokens": K, "tpot_ms": round(tpot, 4), "bytes": sb, "hbm_gbps": round(sb / (tpot * 1e-3) / 1e9, 1),
+                 "frac_of_peak": round(sb / (tpot * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
         return {"workload": "pythia_2b8 full stack, batch-1 greedy decode, hipGraph replay, context 1024", "metric": "tpot_ms",
-                "value": round(tpot, 4), "unit": "ms/token", "bytes": sb, "hbm_gbps": round(sb / (tpot * 1e-3) / 1e9, 1),
-                "frac_of_peak": round(sb / (tpot * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+                "value": round(tpot, 4), "unit": "ms/token", "bytes": sb, "hbm_gbps": first["hbm_gbps"],
+                "frac_of_peak": first["frac_of_peak"], "layer_kernel_us": round(lay_us, 2),
+                "layer_kernel_frac_of_peak": round(layer_bytes(cfg, ctx + 1) / (lay_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                "sweep": [first] + sweep}
 
     def brief(r):
         return {"workload": r["config"]["workload"], "metric": r["metric"], "value": r["value"], "unit": r["unit"],
@@ -307,7 +413,8 @@ def main():
     ap.add_argument("--ctx", type=int, default=2048, help="KV-cache rows already filled when the timed region starts")
     ap.add_argument("--mode", default="fused", choices=["fused", "split"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-also", dest="also", action="store_false", help="skip the short measurements of the other configurations")
+    ap.add_argument("--no-also", dest="also", action="store_false",
+                    help="skip the context sweep, the drop-in per-layer loop and the short measurements of the other configurations")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU (the hot path is a single-GPU batch-1 decode step); "
@@ -330,7 +437,10 @@ def main():
         return bench_llama_batch(args)
     cfg = pkg.PYTHIA_6B9 if args.model == "pythia_6b9" else pkg.PYTHIA_2B8
     K, W = args.steps, args.warmup
-    rows = args.ctx + W + K + 40
+    extras = args.also and args.mode == "fused"
+    sweep_ctx = {"pythia_6b9": [1024, 4096, 8192, 16384], "pythia_2b8": [1024, 2048, 4096]}[args.model]
+    sweep_ctx = [c for c in sweep_ctx if c != args.ctx]
+    rows = max(args.ctx + W + K, (max(sweep_ctx) + 28) if extras else 0) + 40
     t0 = time.perf_counter()
     dec = build_model(cfg, rows, args.ctx, dev, args.mode)
     torch.cuda.synchronize()
@@ -368,8 +478,10 @@ def main():
         wall_ms = (time.perf_counter() - t0) * 1e3
     ev_ms = e0.elapsed_time(e1)
     tpot = wall_ms / K
+    dec.check()                       # raises if any launch of the run raised a device-side failure flag
     state = dec.state.cpu().tolist()
     assert state[1] == args.ctx + W + K, state
+    traffic, traffic_source = recorded_traffic(args.model, args.ctx) if args.mode == "fused" else (None, None)
 
     S_mid = args.ctx + W + K // 2
     sb = step_bytes(cfg, S_mid)
@@ -385,7 +497,7 @@ def main():
                    "mode": args.mode, "context": args.ctx, "hidden": cfg.hidden, "ffn": cfg.ffn, "layers": cfg.n_layers},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.model, args.ctx)) if args.mode == "fused" else None,
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "k_fused (one decoder layer)" if args.mode == "fused" else "stage A+B+C kernels (one decoder layer)",
                      "bytes_per_launch": lb, "launch_us": round(lay_ms * 1e3, 2)},
         "step": {"bytes": sb, "hbm_gbps": round(sb / (tpot * 1e-3) / 1e9, 1),
@@ -393,6 +505,18 @@ def main():
                  "roofline_ms": round(sb / (HBM_PEAK_GBPS * 1e9) * 1e3, 4), "event_ms_per_step": round(ev_ms / K, 4),
                  "lm_head_us": round(sorted(lm_ms)[1] * 1e3, 1)},
     }
+    if extras:
+        with torch.cuda.stream(stream):
+            result["sweep"] = [{"context": args.ctx, "tokens": K, "tpot_ms": round(tpot, 4), "bytes": sb,
+                                "hbm_gbps": result["step"]["hbm_gbps"], "frac_of_peak": result["step"]["frac_of_peak"]}] + \
+                context_sweep(dec, cfg, stream, sweep_ctx)
+        result["sweep"].sort(key=lambda r: r["context"])
+        try:
+            result["drop_in_loop"] = drop_in_loop(args.model, cfg, dec, args.ctx)
+            result["drop_in_loop"]["neox_decoder_tpot_ms"] = round(tpot, 4)
+        except Exception as e:     # noqa: BLE001
+            log(f"[drop_in_loop] failed: {type(e).__name__}: {e}")
+            result["drop_in_loop"] = {"error": f"{type(e).__name__}: {e}"}
     if args.also and args.model == "pythia_6b9":
         del dec
         torch.cuda.empty_cache()
