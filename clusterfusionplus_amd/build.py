@@ -39,10 +39,13 @@ def _run(cmd):
         raise RuntimeError(f"build command failed ({res.returncode}): {' '.join(cmd)}")
 
 
-def build_lib():
+def build_lib(trace: bool = False, out: str = LIB):
+    """libcfpp.so.  `trace`: a profiling build (-DCFPP_TRACE) whose fused kernel stores phase timestamps for
+    `python -m clusterfusionplus_amd.phase_trace`; it is slower by the stores and is never the default."""
     hipcc = os.path.join(ROCM, "bin", "hipcc")
-    _run([hipcc, *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", os.path.join(CSRC, "cfpp_kernels.hip"), "-o", LIB])
-    return LIB
+    extra = ["-DCFPP_TRACE"] if trace else []
+    _run([hipcc, *HIPCC_FLAGS, *extra, f"-I{INCLUDE}", f"-I{CSRC}", os.path.join(CSRC, "cfpp_kernels.hip"), "-o", out])
+    return out
 
 
 def build_ext():
@@ -69,5 +72,12 @@ def build_all():
 
 
 if __name__ == "__main__":
-    build_all()
+    import argparse
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--trace-lib", metavar="PATH", help="only build a profiling variant of libcfpp.so (-DCFPP_TRACE) at PATH")
+    a = ap.parse_args()
+    if a.trace_lib:
+        build_lib(trace=True, out=a.trace_lib)
+    else:
+        build_all()
     sys.exit(0)

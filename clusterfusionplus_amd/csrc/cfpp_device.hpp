@@ -33,7 +33,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
 constexpr int kChunk = 512;            // halfs covered by one wave-wide 16-byte load
-constexpr int kMaxSplit = 64;          // KV splits per head (upper bound; the effective count follows seq_len)
+constexpr int kMaxSplit = 64;          // partial results per head: KV splits (the effective count follows seq_len) + the new token's item
 constexpr int kSplitRows = 64;         // target cache rows per (head, split) item
 constexpr int kMaxWaves = 16;          // waves per workgroup
 constexpr int kRowBatch = 32;          // stage-C rows per workgroup pass
@@ -332,6 +332,8 @@ __device__ __forceinline__ int effective_split(const LayerParams& p, int S) {
     n = n < 1 ? 1 : n;
     return n < p.max_split ? n : p.max_split;
 }
+// items of one head: the KV splits and the new token
+__device__ __forceinline__ int items_per_head(int nsplit) { return nsplit + 1; }
 
 // ------------------------------------------------------------------------------------------------
 // stage A: LayerNorm shared by the workgroup, then row-per-wave streaming GEMV
@@ -740,29 +742,34 @@ __device__ __forceinline__ void rope_coeffs(int d0, int rot, const float* __rest
         }
     }
 }
+// The raw values of a lane's eight dims and of their rotation partners: rope_request issues the loads, rope_finish
+// rotates.  Requests for several vectors (q and k of the new token) issued back to back share one memory round trip.
+struct RopeRaw { float a[8], pr[8]; };
 template <bool PAIRS = false>
-__device__ __forceinline__ void rope_load8(const float* __restrict__ v, int d0, int rot, const RopeCoeffs& rc, bool act,
-                                           float (&out)[8]) {
-    float a[8], pr[8];
+__device__ __forceinline__ void rope_request(const float* __restrict__ v, int d0, int rot, bool act, RopeRaw& r) {
     const int hr = rot >> 1;
     if (act) {
-        ld_agent2(v + d0, a[0], a[1]); ld_agent2(v + d0 + 2, a[2], a[3]);
-        ld_agent2(v + d0 + 4, a[4], a[5]); ld_agent2(v + d0 + 6, a[6], a[7]);
+        ld_agent2(v + d0, r.a[0], r.a[1]); ld_agent2(v + d0 + 2, r.a[2], r.a[3]);
+        ld_agent2(v + d0 + 4, r.a[4], r.a[5]); ld_agent2(v + d0 + 6, r.a[6], r.a[7]);
+        if (!PAIRS) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            if (PAIRS) {
-                pr[j] = a[j ^ 1];                    // the neighbour is one of the lane's own eight dims
-            } else {
+            for (int j = 0; j < 8; ++j) {
                 const int d = d0 + j;
                 const int pd = d < rot ? (d < hr ? d + hr : d - hr) : d;
-                pr[j] = ld_agent(v + pd);
+                r.pr[j] = ld_agent(v + pd);
             }
         }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) out[j] = d0 + j < rot ? a[j] * rc.c[j] + pr[j] * rc.sg[j] : a[j];
     } else {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) out[j] = 0.f;
+        for (int j = 0; j < 8; ++j) { r.a[j] = 0.f; r.pr[j] = 0.f; }
+    }
+}
+template <bool PAIRS = false>
+__device__ __forceinline__ void rope_finish(const RopeRaw& r, int d0, int rot, const RopeCoeffs& rc, bool act, float (&out)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float pr = PAIRS ? r.a[j ^ 1] : r.pr[j];          // GPT-J: the neighbour is one of the lane's own eight dims
+        out[j] = act ? (d0 + j < rot ? r.a[j] * rc.c[j] + pr * rc.sg[j] : r.a[j]) : 0.f;
     }
 }
 __device__ __forceinline__ void raw_load8(const float* __restrict__ v, int d0, bool act, float (&out)[8]) {
@@ -775,7 +782,11 @@ __device__ __forceinline__ void raw_load8(const float* __restrict__ v, int d0, b
     }
 }
 
-// One (head, split) item: the wave's four 16-lane groups take cache rows begin+g, begin+g+4, ...; lane
+// A head's attention is split into nsplit items over its cache rows plus one item for the new token (item index
+// nsplit: it rotates and returns the new K / V row, appends it, and contributes the new token's score and value);
+// attn_items_per_head = nsplit + 1 partial results meet in the merge.  Keeping the new token out of the cache items
+// makes them all alike: the one that used to carry it needed a second dependent memory round trip and ended last.
+// One cache item: the wave's four 16-lane groups take cache rows begin+g, begin+g+4, ...; lane
 // `sub` of a group holds dims 8 sub .. 8 sub + 7 of its row (lanes with 8 sub >= D contribute nothing).
 // A tile is kAttnT rows per group (32 rows per wave).  An item is a chain of dependent memory round
 // trips, so everything that does not depend on this layer's QKV rows is requested ahead of them by
@@ -812,7 +823,7 @@ __device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it
     const int S = sl.S;
     it.head = head; it.sp = sp; it.nsplit = nsplit; it.S = S; it.append_ok = sl.ok;
     const int chunk = (S + nsplit - 1) / nsplit;
-    it.begin = sp * chunk;
+    it.begin = sp < nsplit ? sp * chunk : S;          // item nsplit is the new token: no cache rows
     it.end = (it.begin + chunk < S) ? it.begin + chunk : S;
     it.ntiles = it.begin < it.end ? (it.end - it.begin + kAttnTileRows - 1) / kAttnTileRows : 0;
     if (it.ntiles > 0) attn_load_tile<PAGED>(p, it, it.t0, 0, lane);
@@ -835,23 +846,23 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     const float* __restrict__ raw = p.qkv_raw + (size_t)head * p.qkv_head_stride;
 
     const RopeCoeffs& rc = it.rc;
-    float q[8];
-    rope_load8<PAIRS>(raw, d0, p.rot, rc, act, q);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) q[j] *= p.qscale;
-
     float m = kNegBig, l = 0.f, acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-
-    // the new token: split 0 owns it (appends it, returns it, and seeds its softmax state with it)
-    if (sp == 0 && grp == 0) {
-        float kf[8], vf[8];
-        rope_load8<PAIRS>(raw + p.qkv_k_off, d0, p.rot, rc, act, kf);
-        raw_load8(raw + p.qkv_v_off, d0, act, vf);
+    float q[8];
+    if (sp == nsplit) {
+        // the new token's item: q, k and v of this step, requested together (one round trip); group 0 does the work
+        RopeRaw rq, rk;
+        float vf[8], kf[8];
+        const bool on = act && grp == 0;
+        rope_request<PAIRS>(raw, d0, p.rot, on, rq);
+        rope_request<PAIRS>(raw + p.qkv_k_off, d0, p.rot, on, rk);
+        raw_load8(raw + p.qkv_v_off, d0, on, vf);
+        rope_finish<PAIRS>(rq, d0, p.rot, rc, on, q);
+        rope_finish<PAIRS>(rk, d0, p.rot, rc, on, kf);
         const u32x4 kp = pack8(kf), vp = pack8(vf);
         unpack8(kp, kf); unpack8(vp, vf);      // attend over the fp16 values the cache will hold
-        if (act) {
+        if (on) {
             const size_t o = (size_t)head * D + d0;
             *reinterpret_cast<u32x4*>(p.k_new + o) = kp;
             *reinterpret_cast<u32x4*>(p.v_new + o) = vp;
@@ -866,68 +877,76 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
                 *reinterpret_cast<u32x4*>(p.v_cache + (size_t)S * H + o) = vp;
             }
         }
-        float s = 0.f;
+        if (grp == 0) {
+            float s = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) s += q[j] * kf[j];
-        s = row16_sum(s);
-        m = s; l = 1.f;
+            for (int j = 0; j < 8; ++j) s += q[j] * p.qscale * kf[j];
+            s = row16_sum(s);
+            m = s; l = 1.f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] = vf[j];
-    }
-
-    auto process = [&](const KvTile& kv, int i) {
-        const int r = it.begin + i * kAttnTileRows + grp;
-        float s[kAttnT], mt = m;
-#pragma unroll
-        for (int t = 0; t < kAttnT; ++t) {
-            float kf[8];
-            unpack8(kv.k[t], kf);
-            float d = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) d += q[j] * kf[j];
-            d = row16_sum(d);
-            s[t] = (r + t * 4 < end) ? d : kNegBig;
-            mt = fmaxf(mt, s[t]);
-        }
-        const float alpha = fast_exp2(m - mt);
-        l *= alpha;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] *= alpha;
-#pragma unroll
-        for (int t = 0; t < kAttnT; ++t) {
-            const float pt = (r + t * 4 < end) ? fast_exp2(s[t] - mt) : 0.f;
-            float vf[8];
-            unpack8(kv.v[t], vf);
-            l += pt;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) acc[j] += pt * vf[j];
-        }
-        m = mt;
-    };
-    if (PAGED) {
-        // items of a batched launch can be long: keep two tiles in flight all the way
-        for (int i = 0; i < it.ntiles; i += 2) {
-            process(it.t0, i);
-            __builtin_amdgcn_sched_barrier(0);
-            if (i + 2 < it.ntiles) attn_load_tile<PAGED>(p, it, it.t0, i + 2, lane);
-            __builtin_amdgcn_sched_barrier(0);
-            if (i + 1 < it.ntiles) {
-                process(it.t1, i + 1);
-                __builtin_amdgcn_sched_barrier(0);
-                if (i + 3 < it.ntiles) attn_load_tile<PAGED>(p, it, it.t1, i + 3, lane);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            for (int j = 0; j < 8; ++j) acc[j] = vf[j];
         }
     } else {
-        if (it.ntiles > 0) process(it.t0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        if (it.ntiles > 2) attn_load_tile<PAGED>(p, it, it.t0, 2, lane);     // the third tile travels while the second is reduced
-        __builtin_amdgcn_sched_barrier(0);
-        if (it.ntiles > 1) process(it.t1, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        for (int i = 2; i < it.ntiles; ++i) {
-            if (i != 2) attn_load_tile<PAGED>(p, it, it.t0, i, lane);
-            process(it.t0, i);
+        RopeRaw rq;
+        rope_request<PAIRS>(raw, d0, p.rot, act, rq);
+        rope_finish<PAIRS>(rq, d0, p.rot, rc, act, q);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) q[j] *= p.qscale;
+
+        auto process = [&](const KvTile& kv, int i) {
+            const int r = it.begin + i * kAttnTileRows + grp;
+            float s[kAttnT], mt = m;
+#pragma unroll
+            for (int t = 0; t < kAttnT; ++t) {
+                float kf[8];
+                unpack8(kv.k[t], kf);
+                float d = 0.f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) d += q[j] * kf[j];
+                d = row16_sum(d);
+                s[t] = (r + t * 4 < end) ? d : kNegBig;
+                mt = fmaxf(mt, s[t]);
+            }
+            const float alpha = fast_exp2(m - mt);
+            l *= alpha;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] *= alpha;
+#pragma unroll
+            for (int t = 0; t < kAttnT; ++t) {
+                const float pt = (r + t * 4 < end) ? fast_exp2(s[t] - mt) : 0.f;
+                float vf[8];
+                unpack8(kv.v[t], vf);
+                l += pt;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[j] += pt * vf[j];
+            }
+            m = mt;
+        };
+        if (PAGED) {
+            // items of a batched launch can be long: keep two tiles in flight all the way
+            for (int i = 0; i < it.ntiles; i += 2) {
+                process(it.t0, i);
+                __builtin_amdgcn_sched_barrier(0);
+                if (i + 2 < it.ntiles) attn_load_tile<PAGED>(p, it, it.t0, i + 2, lane);
+                __builtin_amdgcn_sched_barrier(0);
+                if (i + 1 < it.ntiles) {
+                    process(it.t1, i + 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (i + 3 < it.ntiles) attn_load_tile<PAGED>(p, it, it.t1, i + 3, lane);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        } else {
+            if (it.ntiles > 0) process(it.t0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (it.ntiles > 2) attn_load_tile<PAGED>(p, it, it.t0, 2, lane);     // the third tile travels while the second is reduced
+            __builtin_amdgcn_sched_barrier(0);
+            if (it.ntiles > 1) process(it.t1, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            for (int i = 2; i < it.ntiles; ++i) {
+                if (i != 2) attn_load_tile<PAGED>(p, it, it.t0, i, lane);
+                process(it.t0, i);
+            }
         }
     }
 
@@ -958,15 +977,16 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     }
     drain_memory_ops();
     int last = 0;
-    if (lane == 0) last = (__hip_atomic_fetch_add(p.head_cnt + head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nsplit - 1);
+    const int nparts = nsplit + 1;      // the cache items and the new token's item
+    if (lane == 0) last = (__hip_atomic_fetch_add(p.head_cnt + head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nparts - 1);
     last = first_lane(last);
     if (last) {
-        // The last wave of this head merges the splits.  Lane i fetches (m_i, l_i) of split i, so the
+        // The last wave of this head merges the partial results.  Lane i fetches (m_i, l_i) of item i, so the
         // scales come from one round trip; the accumulators (two dims per lane) are fetched kMergeBatch
         // splits at a time, together with the scales, and added in split order.
         const size_t hb = (size_t)head * kMaxSplit;
         float mi = kNegBig, li = 0.f;
-        if (lane < nsplit) ld_agent2(p.part_ml + (hb + lane) * 2, mi, li);
+        if (lane < nparts) ld_agent2(p.part_ml + (hb + lane) * 2, mi, li);
         const int t2 = lane * 2;
         const bool dact = t2 < D;
         constexpr int kMergeBatch = 32;            // splits per memory round trip
@@ -974,7 +994,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
         auto load_acc = [&](int i0) {
 #pragma unroll
             for (int u = 0; u < kMergeBatch; ++u) {
-                const int i = i0 + u < nsplit ? i0 + u : nsplit - 1;
+                const int i = i0 + u < nparts ? i0 + u : nparts - 1;
                 ld_agent2(p.part_acc + (hb + i) * D + (dact ? t2 : 0), a0[u], a1[u]);
             }
         };
@@ -988,11 +1008,11 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
         const float sci = fast_exp2(mi - M);      // scale of split `lane`
         const float lsi = li * sci;
         float L = 0.f, A0 = 0.f, A1 = 0.f;
-        for (int i0 = 0; i0 < nsplit; i0 += kMergeBatch) {
+        for (int i0 = 0; i0 < nparts; i0 += kMergeBatch) {
             if (i0 != 0) load_acc(i0);
 #pragma unroll
             for (int u = 0; u < kMergeBatch; ++u) {
-                const bool in = i0 + u < nsplit;
+                const bool in = i0 + u < nparts;
                 const int i = in ? i0 + u : 0;
                 const float sc = in ? rl(sci, i) : 0.f;
                 L += in ? rl(lsi, i) : 0.f;

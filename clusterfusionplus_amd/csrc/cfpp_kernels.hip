@@ -241,11 +241,11 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_b(LayerParams p) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const SeqLen sl = load_seq_len(p);
-    const int nsplit = effective_split(p, sl.S);
+    const int nsplit = effective_split(p, sl.S), per_head = items_per_head(nsplit);
     const int item = blockIdx.x * kStreamers + wave;
-    if (item < p.heads * nsplit) {
+    if (item < p.heads * per_head) {
         AttnItem it;
-        attn_prefetch(p, it, item / nsplit, item % nsplit, nsplit, sl, lane);
+        attn_prefetch(p, it, item / per_head, item % per_head, nsplit, sl, lane);
         attention_item(p, it, lane, 0, 0);
     }
 }
@@ -332,12 +332,16 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
         ln_coop_load<NCH, kFusedWaves, true>(own, norm_spec(p), wave, lane);
         __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
         if (qkv8 || wave < kStreamers) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
+        trace_mark(p, 14);
+#ifdef CFPP_TRACE
+        trace_value(p, 15, wall_clock64() + (long long)(own.rx[0].x & 0u));     // the wave's chunk of the input row has arrived
+#endif
         ln_coop_finish<NCH, kFusedWaves, true>(own, norm_spec(p), lns, wave, lane);
     }
     const int tag = first_lane(gen) + 1;
     const SeqLen sl = load_seq_len(p);
-    const int nsplit = effective_split(p, sl.S);
-    const int nitems = p.heads * nsplit;
+    const int nsplit = effective_split(p, sl.S), per_head = items_per_head(nsplit);
+    const int nitems = p.heads * per_head;
     const int attn_count = nitems > b ? (nitems - b + G - 1) / G : 0;
     trace_mark(p, 1);
     // Counting an arrival device-wide is two dependent atomic round trips for the wave that does it, and a
@@ -423,10 +427,11 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
             ln_fetch<NCH>(lns, 0, lane, xq);
             qkv_rows<NCH, EX>(p, xq, qw, lane, t0, hpark);
             event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
+            trace_mark(p, 2);
         }
         if (hw < attn_count) {
             AttnItem it;
-            attn_prefetch(p, it, (b + hw * G) / nsplit, (b + hw * G) % nsplit, nsplit, sl, lane);
+            attn_prefetch(p, it, (b + hw * G) / per_head, (b + hw * G) % per_head, nsplit, sl, lane);
             event_wait(p.mbox, kBarQkv, tag, status);
             __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
             trace_mark(p, 3);
@@ -1074,11 +1079,11 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gemv_t(GemvT a) {
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_b_pairs(LayerParams p) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
     const SeqLen sl = load_seq_len(p);
-    const int nsplit = effective_split(p, sl.S);
+    const int nsplit = effective_split(p, sl.S), per_head = items_per_head(nsplit);
     const int item = blockIdx.x * kStreamers + wave;
-    if (item < p.heads * nsplit) {
+    if (item < p.heads * per_head) {
         AttnItem it;
-        attn_prefetch<false, true>(p, it, item / nsplit, item % nsplit, nsplit, sl, lane);
+        attn_prefetch<false, true>(p, it, item / per_head, item % per_head, nsplit, sl, lane);
         attention_item<false, true>(p, it, lane, 0, 0);
     }
 }
@@ -1096,11 +1101,12 @@ struct BatchAttn {
 __global__ __launch_bounds__(kStreamers * 64) void k_batch_attn(LayerParams p, BatchAttn b) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
     const int item = blockIdx.x * kStreamers + wave;
-    const int per_seq = p.heads * p.max_split;
+    const int slots = items_per_head(p.max_split);          // item slots per head: the KV splits in use, the new token, spares
+    const int per_seq = p.heads * slots;
     const int seq = item / per_seq;
     if (seq >= b.batch) return;
     const int rem = item - seq * per_seq;
-    const int head = rem / p.max_split, sp = rem - head * p.max_split;
+    const int head = rem / slots, sp = rem - head * slots;
     const int start = b.indptr[seq];
     int S = b.indptr[seq + 1] - 1 - start;
     if (S < 0) {
@@ -1108,7 +1114,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_attn(LayerParams p, B
         return;
     }
     const int nsplit = effective_split(p, S);
-    if (sp >= nsplit) return;
+    if (sp > nsplit) return;               // sp == nsplit is the new token's item
     LayerParams q = p;
     q.kv_rows = b.indices + start;
     q.k_cache = reinterpret_cast<half_t*>(b.k_ptrs[b.layer_id]);
@@ -1443,9 +1449,9 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 // KV splits per head at most: `item_waves` attention waves per workgroup of the fused launch get an item
 int split_cap(int heads, int item_waves) {
-    int ms = kMaxSplit;
+    int ms = kMaxSplit - 1;               // + the new token's item
     const int per_head = fused_grid() * item_waves / (heads > 0 ? heads : 1);
-    if (ms > per_head) ms = per_head < 1 ? 1 : per_head;
+    if (ms > per_head - 1) ms = per_head < 2 ? 1 : per_head - 1;     // one of a head's item slots is the new token's
     return ms;
 }
 int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_neox_io* io, void* workspace,
@@ -1528,7 +1534,9 @@ int run_split(const Plan& pl, LayerParams& p, int seq_hint, hipStream_t st);
 int run_layer(const Plan& pl, LayerParams& p, int mode, int seq_hint, hipStream_t st) {
     if (mode == CFPP_MODE_SPLIT) return run_split(pl, p, seq_hint, st);
     const int grid = fused_grid();
-    if (p.heads > grid * kStreamers || !fused_fits(pl, p, grid)) return run_split(pl, p, seq_hint, st);
+    // every attention wave of the one-launch kernel takes at most one item
+    if ((long long)p.heads * (p.max_split + 1) > (long long)grid * kStreamers || !fused_fits(pl, p, grid))
+        return run_split(pl, p, seq_hint, st);
     return launch_fused(pl, p, grid, st);
 }
 
@@ -1536,7 +1544,7 @@ int run_split(const Plan& pl, LayerParams& p, int seq_hint, hipStream_t st) {
     const int grid = grid_for_streaming(pl);
     int rc = launch_stage_a(pl, p, grid, st);
     if (rc) return rc;
-    const int bgrid = (p.heads * split_bound(seq_hint, p.max_split) + kStreamers - 1) / kStreamers;
+    const int bgrid = (p.heads * (split_bound(seq_hint, p.max_split) + 1) + kStreamers - 1) / kStreamers;
     hipLaunchKernelGGL(k_stage_b, dim3(bgrid), dim3(kStreamers * 64), 0, st, p);
     if ((rc = launch_check())) return rc;
     return launch_stage_c(pl, p, grid, st);
@@ -1829,7 +1837,7 @@ int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t
     };
     // the QKV launch normalises the input row on its way in (a separate norm launch was measured slower)
     if ((rc = gemv(h(a->w_qkv), 3, h(a->input), h(a->rms_w), p.qkv_raw, nullptr))) return rc;
-    const int bgrid = (p.heads * split_bound(a->seq_len, p.max_split) + kStreamers - 1) / kStreamers;
+    const int bgrid = (p.heads * (split_bound(a->seq_len, p.max_split) + 1) + kStreamers - 1) / kStreamers;
     hipLaunchKernelGGL(k_stage_b_pairs, dim3(bgrid), dim3(kStreamers * 64), 0, st, p);
     if ((rc = (int)hipGetLastError())) return rc;
     return gemv(h(a->w_o), 1, p.attn_vec, nullptr, nullptr, reinterpret_cast<half_t*>(a->output));
@@ -1964,7 +1972,7 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
     b.v_ptrs = reinterpret_cast<const unsigned long long*>(a->v_cache_ptrs);
     b.positions = reinterpret_cast<const long long*>(a->positions);
     b.cos_sin = a->cos_sin;
-    const long long items = (long long)a->batch * d.heads * p.max_split;
+    const long long items = (long long)a->batch * d.heads * (p.max_split + 1);
     const int agrid = (int)((items + kStreamers - 1) / kStreamers);
     hipLaunchKernelGGL(k_batch_attn, dim3(agrid), dim3(kStreamers * 64), 0, st, p, b);
     if ((rc = (int)hipGetLastError())) return rc;

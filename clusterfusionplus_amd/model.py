@@ -92,6 +92,7 @@ class NeoxDecoder:
                  k_caches: List[torch.Tensor], v_caches: List[torch.Tensor], mode: str = "fused"):
         from . import _clusterfusion as native
         self.cfg = cfg
+        self._layers, self._k_caches, self._v_caches = list(layers), list(k_caches), list(v_caches)   # keep the storage alive
         rows = k_caches[0].shape[0]
         self.cos, self.sin = rope_tables(rows, cfg.rotary_dim, cfg.rope_base, device=embed.device)
         packed = [[w[k].reshape(-1) if w[k].dim() == 1 else w[k] for k in layer_tensor_order] for w in layers]

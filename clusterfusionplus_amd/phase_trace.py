@@ -1,0 +1,95 @@
+"""Phase timeline of the fused decoder-layer kernel inside a whole-model decode step.
+
+Needs a profiling build of the HIP library (`python -m clusterfusionplus_amd.build --trace-lib PATH`, then PATH in
+place of libcfpp.so): its fused kernel stores a 100 MHz timestamp per wave at every phase boundary.  This tool runs a
+synthetic model of the given shape, records one eager step, and prints per phase the median over the layers of the
+mean / earliest / latest time (microseconds from the kernel's first wave) over all workgroups.
+
+    python -m clusterfusionplus_amd.phase_trace --model pythia_2b8 --ctx 1024
+"""
+import argparse
+import sys
+
+import numpy as np
+import torch
+
+# slot -> (label, which waves report it)
+SLOTS = [(0, "kernel entry", "all"), (14, "LayerNorm inputs and first weight tile requested", "all"), (15, "own chunk of the input row arrived", "all"),
+         (1, "LayerNorm done", "all"), (2, "own QKV rows stored, QKV arrival counted", "streaming"),
+         (2, "own QKV rows stored, QKV arrival counted", "attention"),
+         (3, "QKV event seen, attention item begins", "attention"), (4, "attention item done (head merged by its last split)", "attention"),
+         (12, "own MLP-up phase 0 rows stored", "streaming"), (5, "own MLP-up phase 1 rows stored", "streaming"),
+         (6, "MLP-up phase 0 event seen (down phase 0 may read)", "streaming"), (13, "MLP-up phase 1 event seen (down phase 1 may read)", "streaming"),
+         (7, "heads event seen (O rows may read)", "attention"), (9, "stage C begins", "all"), (10, "stage C done: rows reduced and stored", "all")]
+
+
+def synthetic_decoder(cfg, rows, device):
+    from . import NeoxDecoder
+    torch.manual_seed(0)
+    H, F = cfg.hidden, cfg.ffn
+
+    def rn(shape, std, mean=0.0):
+        return torch.empty(shape, dtype=torch.float16, device=device).normal_(mean, std)
+    layers = [{"ln_w": rn((H,), 0.02, 1.0), "ln_b": rn((H,), 0.01), "w_qkv": rn((3 * H, H), 0.02), "b_qkv": rn((3 * H,), 0.01),
+               "w_o": rn((H, H), 0.02), "b_o": rn((H,), 0.01), "post_ln_w": rn((H,), 0.02, 1.0), "post_ln_b": rn((H,), 0.01),
+               "w_up": rn((F, H), 0.02), "b_up": rn((F,), 0.01), "w_down": rn((H, F), 0.02), "b_down": rn((H,), 0.01)}
+              for _ in range(cfg.n_layers)]
+    return NeoxDecoder(cfg, layers, rn((cfg.vocab, H), 1.0), rn((H,), 0.02, 1.0), rn((H,), 0.01), rn((cfg.vocab, H), 0.02),
+                       [rn((rows, H), 1.0) for _ in range(cfg.n_layers)], [rn((rows, H), 1.0) for _ in range(cfg.n_layers)])
+
+
+def main():
+    from . import PYTHIA_2B8, PYTHIA_6B9, debug_set_trace
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8"])
+    ap.add_argument("--ctx", type=int, default=2048)
+    ap.add_argument("--raw", help="also save the raw timestamps of the last layer ([workgroup][wave][slot]) as .npy")
+    a = ap.parse_args()
+    cfg = PYTHIA_6B9 if a.model == "pythia_6b9" else PYTHIA_2B8
+    dev = "cuda:0"
+    dec = synthetic_decoder(cfg, a.ctx + 64, dev)
+    dec.set_state(11, a.ctx)
+    for _ in range(3):
+        dec.step()
+    torch.cuda.synchronize()
+    lay, _lm, _tot = dec.profile_step()
+    print(f"{a.model}, context {a.ctx}: fused layer kernel {np.median(lay) * 1e3:.1f} us (median of {len(lay)} layers, HIP events, "
+          "profiling build)")
+    # the trace buffer holds one launch: record the layers of one step one at a time through the per-layer op
+    tr = torch.zeros(1024 * 16 * 16, dtype=torch.int64, device=dev)
+    debug_set_trace(tr)          # raises unless the library is a profiling build
+    per_layer = []
+    import clusterfusionplus_amd as pkg
+    op = pkg.neox_decoder_layer
+    # re-run single layers with their own weights (cold: 32 different weight sets in turn)
+    x = torch.randn(1, cfg.hidden, device=dev).half()
+    cos, sin = dec.cos[a.ctx:a.ctx + 1].contiguous(), dec.sin[a.ctx:a.ctx + 1].contiguous()
+    for l, w in enumerate(dec._layers):
+        tr.zero_()
+        op(cfg.hidden, cfg.heads, cfg.head_dim, cfg.rotary_dim, cfg.ffn, cfg.eps, False, x, w["w_qkv"], w["b_qkv"], w["w_o"], w["b_o"],
+           dec._k_caches[l], dec._v_caches[l], w["ln_w"], w["ln_b"], cos, sin, w["post_ln_w"], w["post_ln_b"], w["w_up"], w["b_up"],
+           w["w_down"], w["b_down"], a.ctx)
+        torch.cuda.synchronize()
+        per_layer.append(tr.cpu().numpy().reshape(1024, 16, 16)[:256, :8].astype(np.float64))
+    debug_set_trace(None)
+    if a.raw:
+        np.save(a.raw, per_layer[-1])
+    rows = {}
+    for raw in per_layer[2:]:
+        t0 = raw[:, :, 0][raw[:, :, 0] > 0].min()
+        us = (raw - t0) / 100.0
+        for slot, label, who in SLOTS:
+            sl = {"all": slice(0, 8), "streaming": slice(0, 4), "attention": slice(4, 8)}[who]
+            col = us[:, sl, slot][raw[:, sl, slot] > 0]
+            if col.size:
+                rows.setdefault((slot, who), []).append((col.mean(), col.min(), np.percentile(col, 50), col.max()))
+    print(f"{'phase boundary (us from the first wave; median over layers of ...)':84s} {'mean':>7s} {'first':>7s} {'median':>7s} {'last':>7s}")
+    for slot, label, who in SLOTS:
+        if (slot, who) in rows:
+            m = np.median(np.array(rows[(slot, who)]), axis=0)
+            print(f"{label + ' [' + who + ' waves]':84s} {m[0]:7.2f} {m[1]:7.2f} {m[2]:7.2f} {m[3]:7.2f}")
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
