@@ -42,6 +42,9 @@ constexpr int kStreamers = 4;          // streaming waves per workgroup: one per
 constexpr int kUpPhases = 2;           // the MLP intermediate is produced and consumed in this many phases
 constexpr float kNegBig = -1.0e30f;
 constexpr int kSpinLimit = 1 << 20;    // bounded device-side waits (order of a second)
+constexpr int kHeadCntStride = 16;     // ints between the arrival counters of two heads: returning atomics of different
+                                       // heads must not meet in one cache line (they serialise at the memory side; with
+                                       // all 32 counters in one line the items of a Pythia-2.8B layer ended 1 us later)
 
 enum : int { kStatusSpin = 1, kStatusSeq = 2 };
 // Slots of LayerParams::bar.  The event counters reset themselves (the arrival that completes a count
@@ -87,7 +90,7 @@ struct LayerParams {
     half_t* inter;      // [F] fp16: gelu(W_up ln2(x) + b_up)
     float* part_ml;     // [heads][kMaxSplit][2] running max (log2 domain) and denominator
     float* part_acc;    // [heads][kMaxSplit][D]
-    int* head_cnt;      // [heads] arrival counters, self-resetting
+    int* head_cnt;      // [heads][kHeadCntStride] arrival counters (one 64-byte line per head), self-resetting
     int* bar;           // device-wide counters, see BarSlot
     int* grp;           // [events][kEventGroups] group counters, one 64-byte line each
     int* mbox;          // [kMaxGrid][kMailboxInts] event flags, one line per workgroup
@@ -978,7 +981,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     drain_memory_ops();
     int last = 0;
     const int nparts = nsplit + 1;      // the cache items and the new token's item
-    if (lane == 0) last = (__hip_atomic_fetch_add(p.head_cnt + head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nparts - 1);
+    if (lane == 0) last = (__hip_atomic_fetch_add(p.head_cnt + head * kHeadCntStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nparts - 1);
     last = first_lane(last);
     if (last) {
         // The last wave of this head merges the partial results.  Lane i fetches (m_i, l_i) of item i, so the
@@ -1024,7 +1027,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
             const half2_t o = {(half_t)(A0 / L), (half_t)(A1 / L)};
             st_agent(reinterpret_cast<uint32_t*>(p.attn_vec + (size_t)head * D + t2), as_u32(o));
         }
-        if (lane == 0) __hip_atomic_store(p.head_cnt + head, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) __hip_atomic_store(p.head_cnt + head * kHeadCntStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (nwg_to_signal > 0) {
             // count the head; the wave that completes the count tells every workgroup
             drain_memory_ops();

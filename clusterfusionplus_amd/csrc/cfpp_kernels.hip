@@ -1128,7 +1128,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_attn(LayerParams p, B
     q.v_new += (size_t)seq * p.H;
     q.part_ml += (size_t)seq * p.heads * kMaxSplit * 2;
     q.part_acc += (size_t)seq * p.heads * kMaxSplit * p.D;
-    q.head_cnt += (size_t)seq * p.heads;
+    q.head_cnt += (size_t)seq * p.heads * kHeadCntStride;
     AttnItem it;
     attn_prefetch<true>(q, it, head, sp, nsplit, SeqLen{S, true}, lane);
     attention_item<true>(q, it, lane, 0, 0);
@@ -1241,7 +1241,7 @@ WorkspaceLayout workspace_layout(const cfpp_neox_dims& d) {
     w.inter = take((size_t)d.ffn * 2);
     w.part_ml = take((size_t)d.heads * kMaxSplit * 2 * 4);
     w.part_acc = take((size_t)d.heads * kMaxSplit * d.head_dim * 4);
-    w.head_cnt = take((size_t)d.heads * 4);
+    w.head_cnt = take((size_t)d.heads * kHeadCntStride * 4);
     w.bar = take(64);
     w.grp = take((size_t)(kBarExit + 1) * kEventGroups * kMailboxInts * 4);
     w.mbox = take((size_t)kMaxGrid * kMailboxInts * 4);
@@ -1570,7 +1570,7 @@ BatchLayout batch_layout(const cfpp_neox_dims& d, int batch) {
     w.v_new = take(B * H * 2);
     w.part_ml = take(B * d.heads * kMaxSplit * 2 * 4);
     w.part_acc = take(B * d.heads * kMaxSplit * (size_t)d.head_dim * 4);
-    w.head_cnt = take(B * d.heads * 4);
+    w.head_cnt = take(B * d.heads * kHeadCntStride * 4);
     w.bar = take(64 * 4);
     w.total = off;
     return w;
