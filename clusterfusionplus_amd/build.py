@@ -48,6 +48,39 @@ def build_lib(trace: bool = False, out: str = LIB):
     return out
 
 
+def resource_report(out=None):
+    """Compiles the HIP library with the compiler's kernel-resource-usage remarks and returns one line per kernel:
+    VGPRs, AGPRs, scratch bytes per lane (register spills), static LDS bytes per workgroup, waves per SIMD."""
+    import re
+    import tempfile
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    with tempfile.TemporaryDirectory() as tmp:
+        cmd = [hipcc, *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", f"-I{INCLUDE}", f"-I{CSRC}",
+               os.path.join(CSRC, "cfpp_kernels.hip"), "-o", os.path.join(tmp, "libcfpp.so")]
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("resource report: compilation failed\n" + res.stdout[-2000:])
+    rows = []
+    for block in re.split(r"remark: [^\n]*Function Name: ", res.stdout)[1:]:
+        name = block.split()[0]
+        nice = subprocess.run(["c++filt", name], stdout=subprocess.PIPE, text=True).stdout.strip() or name
+        nice = nice.replace("(anonymous namespace)::", "").replace("void ", "")
+        nice = re.sub(r"\(.*\)$", "", nice)
+
+        def g(key):
+            m = re.search(key + r": (\S+)", block)
+            return m.group(1) if m else "?"
+        rows.append((nice, g("VGPRs"), g("AGPRs"), g(r"ScratchSize \[bytes/lane\]"), g(r"LDS Size \[bytes/block\]"),
+                     g(r"Occupancy \[waves/SIMD\]")))
+    lines = [f"{'kernel':44s} {'VGPRs':>6s} {'AGPRs':>6s} {'scratch B/lane':>15s} {'LDS B/workgroup':>16s} {'waves/SIMD':>11s}"]
+    lines += [f"{n[:44]:44s} {v:>6s} {a:>6s} {sc:>15s} {l:>16s} {o:>11s}" for n, v, a, sc, l, o in rows]
+    text = "\n".join(lines)
+    if out:
+        with open(out, "w") as f:
+            f.write(text + "\n")
+    return text
+
+
 def build_ext():
     import torch
     from torch.utils import cpp_extension as ce
@@ -75,8 +108,12 @@ if __name__ == "__main__":
     import argparse
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--trace-lib", metavar="PATH", help="only build a profiling variant of libcfpp.so (-DCFPP_TRACE) at PATH")
+    ap.add_argument("--resource-report", action="store_true",
+                    help="only print registers, scratch, LDS and occupancy of every kernel (compiler remarks)")
     a = ap.parse_args()
-    if a.trace_lib:
+    if a.resource_report:
+        print(resource_report())
+    elif a.trace_lib:
         build_lib(trace=True, out=a.trace_lib)
     else:
         build_all()

@@ -425,8 +425,13 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
             RowPark hpark{lds.park_attn[hw], 0};
             half2_t xq[NCH][4];
             ln_fetch<NCH>(lns, 0, lane, xq);
+            // ahead of the streaming wave on the same SIMD: that one goes on to its MLP-up tiles as soon as its own
+            // QKV rows are done, and would keep pushing this wave's last QKV tile, which every attention item waits for,
+            // further back
+            __builtin_amdgcn_s_setprio(2);
             qkv_rows<NCH, EX>(p, xq, qw, lane, t0, hpark);
             event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
+            __builtin_amdgcn_s_setprio(0);
             trace_mark(p, 2);
         }
         if (hw < attn_count) {
