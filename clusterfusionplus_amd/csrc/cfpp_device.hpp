@@ -789,6 +789,8 @@ __device__ __forceinline__ void raw_load8(const float* __restrict__ v, int d0, b
 // nsplit: it rotates and returns the new K / V row, appends it, and contributes the new token's score and value);
 // attn_items_per_head = nsplit + 1 partial results meet in the merge.  Keeping the new token out of the cache items
 // makes them all alike: the one that used to carry it needed a second dependent memory round trip and ended last.
+// (The batched kernel, PAGED, keeps the new token in split 0, with its k and v requested together with q: it has a few
+// splits per head only, sized to fill the device exactly once, and an extra item per head would start a second round.)
 // One cache item: the wave's four 16-lane groups take cache rows begin+g, begin+g+4, ...; lane
 // `sub` of a group holds dims 8 sub .. 8 sub + 7 of its row (lanes with 8 sub >= D contribute nothing).
 // A tile is kAttnT rows per group (32 rows per wave).  An item is a chain of dependent memory round
@@ -826,7 +828,7 @@ __device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it
     const int S = sl.S;
     it.head = head; it.sp = sp; it.nsplit = nsplit; it.S = S; it.append_ok = sl.ok;
     const int chunk = (S + nsplit - 1) / nsplit;
-    it.begin = sp < nsplit ? sp * chunk : S;          // item nsplit is the new token: no cache rows
+    it.begin = sp < nsplit ? sp * chunk : S;          // item nsplit (if it exists) is the new token: no cache rows
     it.end = (it.begin + chunk < S) ? it.begin + chunk : S;
     it.ntiles = it.begin < it.end ? (it.end - it.begin + kAttnTileRows - 1) / kAttnTileRows : 0;
     if (it.ntiles > 0) attn_load_tile<PAGED>(p, it, it.t0, 0, lane);
@@ -853,15 +855,18 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.f;
     float q[8];
-    if (sp == nsplit) {
-        // the new token's item: q, k and v of this step, requested together (one round trip); group 0 does the work
+    constexpr bool OWN_ITEM = !PAGED;       // the new token is item nsplit of its head; otherwise split 0 carries it
+    // q, k and v of this step for the wave that handles the new token, requested together (one round trip); group 0
+    // does the work: rotates, returns and appends the new row, and seeds its softmax state with the new token
+    // (every group gets its unscaled q from the same request)
+    auto new_token = [&]() {
         RopeRaw rq, rk;
         float vf[8], kf[8];
         const bool on = act && grp == 0;
-        rope_request<PAIRS>(raw, d0, p.rot, on, rq);
+        rope_request<PAIRS>(raw, d0, p.rot, act, rq);
         rope_request<PAIRS>(raw + p.qkv_k_off, d0, p.rot, on, rk);
         raw_load8(raw + p.qkv_v_off, d0, on, vf);
-        rope_finish<PAIRS>(rq, d0, p.rot, rc, on, q);
+        rope_finish<PAIRS>(rq, d0, p.rot, rc, act, q);
         rope_finish<PAIRS>(rk, d0, p.rot, rc, on, kf);
         const u32x4 kp = pack8(kf), vp = pack8(vf);
         unpack8(kp, kf); unpack8(vp, vf);      // attend over the fp16 values the cache will hold
@@ -889,12 +894,21 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
 #pragma unroll
             for (int j = 0; j < 8; ++j) acc[j] = vf[j];
         }
+    };
+    if (OWN_ITEM && sp == nsplit) {
+        new_token();
     } else {
-        RopeRaw rq;
-        rope_request<PAIRS>(raw, d0, p.rot, act, rq);
-        rope_finish<PAIRS>(rq, d0, p.rot, rc, act, q);
+        if (!OWN_ITEM && sp == 0) {
+            new_token();          // split 0 of the batched kernel carries the new token
 #pragma unroll
-        for (int j = 0; j < 8; ++j) q[j] *= p.qscale;
+            for (int j = 0; j < 8; ++j) q[j] *= p.qscale;
+        } else {
+            RopeRaw rq;
+            rope_request<PAIRS>(raw, d0, p.rot, act, rq);
+            rope_finish<PAIRS>(rq, d0, p.rot, rc, act, q);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] *= p.qscale;
+        }
 
         auto process = [&](const KvTile& kv, int i) {
             const int r = it.begin + i * kAttnTileRows + grp;
@@ -980,7 +994,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     }
     drain_memory_ops();
     int last = 0;
-    const int nparts = nsplit + 1;      // the cache items and the new token's item
+    const int nparts = OWN_ITEM ? nsplit + 1 : nsplit;      // the cache items and the new token's item
     if (lane == 0) last = (__hip_atomic_fetch_add(p.head_cnt + head * kHeadCntStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nparts - 1);
     last = first_lane(last);
     if (last) {

@@ -1106,7 +1106,7 @@ struct BatchAttn {
 __global__ __launch_bounds__(kStreamers * 64) void k_batch_attn(LayerParams p, BatchAttn b) {
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
     const int item = blockIdx.x * kStreamers + wave;
-    const int slots = items_per_head(p.max_split);          // item slots per head: the KV splits in use, the new token, spares
+    const int slots = p.max_split;                          // item slots per head (split 0 carries the new token)
     const int per_seq = p.heads * slots;
     const int seq = item / per_seq;
     if (seq >= b.batch) return;
@@ -1119,7 +1119,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_attn(LayerParams p, B
         return;
     }
     const int nsplit = effective_split(p, S);
-    if (sp > nsplit) return;               // sp == nsplit is the new token's item
+    if (sp >= nsplit) return;
     LayerParams q = p;
     q.kv_rows = b.indices + start;
     q.k_cache = reinterpret_cast<half_t*>(b.k_ptrs[b.layer_id]);
@@ -1977,7 +1977,7 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
     b.v_ptrs = reinterpret_cast<const unsigned long long*>(a->v_cache_ptrs);
     b.positions = reinterpret_cast<const long long*>(a->positions);
     b.cos_sin = a->cos_sin;
-    const long long items = (long long)a->batch * d.heads * (p.max_split + 1);
+    const long long items = (long long)a->batch * d.heads * p.max_split;
     const int agrid = (int)((items + kStreamers - 1) / kStreamers);
     hipLaunchKernelGGL(k_batch_attn, dim3(agrid), dim3(kStreamers * 64), 0, st, p, b);
     if ((rc = (int)hipGetLastError())) return rc;
