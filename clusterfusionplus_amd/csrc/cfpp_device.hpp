@@ -51,13 +51,14 @@ enum : int { kStatusSpin = 1, kStatusSeq = 2 };
 // stores zero); flags are not reset at all: a launch raises a flag by writing its tag, the launch
 // generation read from kBarGen plus one, and the last workgroup to leave stores that tag back.
 enum BarSlot : int {
-    kBarQkv = 0,      // streaming waves that have written their QKV rows
-    kBarUp = 1,       // kBarUp + g: streaming waves that have written their MLP-up rows of phase g (kUpPhases slots)
-    kBarHeads = 3,    // heads whose attention output is merged
-    kBarExit = 4,     // workgroups that have finished
-    kBarStatus = 5,   // failure flags (kStatusSpin, kStatusSeq); never reset by the kernels
-    kBarGen = 6       // launch generation
+    kBarQkv = 0,                      // streaming waves that have written their QKV rows
+    kBarUp = 1,                       // kBarUp + g: streaming waves that have written their MLP-up rows of phase g (kUpPhases slots)
+    kBarHeads = kBarUp + kUpPhases,   // heads whose attention output is merged
+    kBarExit = kBarHeads + 1,         // workgroups that have finished
+    kBarStatus = kBarExit + 1,        // failure flags (kStatusSpin, kStatusSeq); never reset by the kernels
+    kBarGen = kBarStatus + 1          // launch generation
 };
+static_assert(kBarGen < 16, "the slots are the ints of one 64-byte line");
 
 struct LayerParams {
     int H, heads, D, rot, F;
@@ -1176,6 +1177,23 @@ struct DownPhase {
     }
 };
 
+// The MLP-down phases g = G .. kUpPhases-1 of the rows [b0, b1) of one streaming wave, one after the other; phase g
+// waits for down_ready(g) (on the first row batch only) after its first weight tile has been requested.  A phase without
+// chunk slots (small geometries have fewer slots than phases) only passes its wait.
+template <int CPD, int G, class DownReady>
+__device__ __forceinline__ void down_phases(const StageC& c, int ks, int lane, int b0, int b1, StageCShared& sh, bool first,
+                                            DownReady&& down_ready) {
+    typedef DownPhase<down_slot_begin(CPD, G), down_slot_end(CPD, G)> P;
+    if constexpr (P::N > 0) {
+        typename P::Tile t;
+        P::load(c, ks, lane, t, b0, b1);
+        P::run(c, ks, lane, b0, b1, sh.red_down[G], t, [&] { if (first) down_ready(G); }, [] {});
+    } else {
+        if (first) down_ready(G);
+    }
+    if constexpr (G + 1 < kUpPhases) down_phases<CPD, G + 1>(c, ks, lane, b0, b1, sh, first, down_ready);
+}
+
 // Stage C for the rows of workgroup `wg`, as two independent GEMVs whose results meet in LDS:
 //   MLP down   K-split over the kStreamers streaming waves (wave ks owns the 512-half chunks ks, ks+4, ...
 //              of W2 and x2, at most CPD of them, activation slices in registers), RPI rows per tile, two
@@ -1195,21 +1213,7 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
     bool first = true;
     for (int b0 = r0; b0 < r1; b0 += kRowBatch) {
         const int b1 = (b0 + kRowBatch < r1) ? b0 + kRowBatch : r1;
-        if (streamer && c.K2 > 0) {
-            static_assert(kUpPhases == 2, "two phases are written out below");
-            typedef DownPhase<down_slot_begin(CPD, 0), down_slot_end(CPD, 0)> P0;
-            typedef DownPhase<down_slot_begin(CPD, 1), down_slot_end(CPD, 1)> P1;
-            typename P0::Tile t0;
-            P0::load(c, ks, lane, t0, b0, b1);
-            if constexpr (P1::N > 0) {
-                typename P1::Tile t1;
-                P0::run(c, ks, lane, b0, b1, sh.red_down[0], t0, [&] { if (first) down_ready(0); }, [] {});
-                P1::load(c, ks, lane, t1, b0, b1);
-                P1::run(c, ks, lane, b0, b1, sh.red_down[1], t1, [&] { if (first) down_ready(1); }, [] {});
-            } else {
-                P0::run(c, ks, lane, b0, b1, sh.red_down[0], t0, [&] { if (first) { down_ready(0); down_ready(1); } }, [] {});
-            }
-        }
+        if (streamer && c.K2 > 0) down_phases<CPD, 0>(c, ks, lane, b0, b1, sh, first, down_ready);
         if (o_index >= 0 && c.K1 > 0) {
             // up to kORows rows of this wave are requested before the attention vector is waited for, so that
             // only one more round trip (the vector itself) follows the wait
