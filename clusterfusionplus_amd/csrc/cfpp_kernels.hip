@@ -49,7 +49,7 @@ __device__ __forceinline__ void qkv_rows(const LayerParams& p, const half2_t (&x
                                          RowTile<NCH, StageARpi<NCH>::value>& pre, RowPark& park) {
     constexpr int RPI = StageARpi<NCH>::value;
     const int first = rw.first, step = rw.step;
-    gemv_tiles<NCH, RPI, EX>(
+    gemv_tiles<NCH, RPI, EX, RollTiles<NCH>::value>(
         p.w_qkv, p.H, rw.end, rw.sit, rw.ntiles, [=](int t) { return first + t * step; }, x1, lane, pre, park,
         [&](const RowPark& pk, int k0) {
             if (lane < pk.n) {
@@ -74,7 +74,7 @@ template <int NCH, bool EX>
 __device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], const RowWalk& rw, int lane,
                                         RowTile<NCH, kUpRpi>& pre, RowPark& park) {
     const int first = rw.first, step = rw.step;
-    gemv_tiles<NCH, kUpRpi, EX>(
+    gemv_tiles<NCH, kUpRpi, EX, RollTiles<NCH>::value>(
         p.w_up, p.H, rw.end, rw.sit, rw.ntiles, [=](int t) { return first + t * step; }, x2, lane, pre, park,
         [&](const RowPark& pk, int k0) {
             if (lane < pk.n) {
@@ -116,7 +116,7 @@ __device__ __forceinline__ void qkv_team_rows(const LayerParams& p, const half2_
 template <int NCH, bool EX>
 __device__ __forceinline__ void up_team_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], const TileTeam& tm, int lane,
                                              TeamTiles<NCH, kUpRpi>& tt, RowParkIds& park) {
-    gemv_team<NCH, kUpRpi, EX>(p.w_up, p.H, tm, x2, lane, tt, park, [&](const RowParkIds& pk) {
+    gemv_team<NCH, kUpRpi, EX, RollTiles<NCH>::value>(p.w_up, p.H, tm, x2, lane, tt, park, [&](const RowParkIds& pk) {
         if (lane < pk.n) {
             const int row = pk.row[lane];
             if (row >= 0) st_agent(p.inter + row, (half_t)gelu_tanh(pk.slot[lane] + (float)p.b_up[row]));

@@ -43,7 +43,7 @@ def main():
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8"])
     ap.add_argument("--ctx", type=int, default=2048)
-    ap.add_argument("--raw", help="also save the raw timestamps of the last layer ([workgroup][wave][slot]) as .npy")
+    ap.add_argument("--raw", help="also save the raw timestamps of every layer ([layer][workgroup][wave][slot]) as .npy")
     a = ap.parse_args()
     cfg = PYTHIA_6B9 if a.model == "pythia_6b9" else PYTHIA_2B8
     dev = "cuda:0"
@@ -73,7 +73,7 @@ def main():
         per_layer.append(tr.cpu().numpy().reshape(1024, 16, 16)[:256, :8].astype(np.float64))
     debug_set_trace(None)
     if a.raw:
-        np.save(a.raw, per_layer[-1])
+        np.save(a.raw, np.stack(per_layer))
     rows = {}
     for raw in per_layer[2:]:
         t0 = raw[:, :, 0][raw[:, :, 0] > 0].min()
