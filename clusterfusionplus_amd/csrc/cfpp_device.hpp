@@ -244,6 +244,10 @@ __device__ __forceinline__ float silu(float x) { return x / (1.0f + __builtin_am
 constexpr int kMailboxInts = 16;       // one 64-byte line per workgroup
 constexpr int kMaxGrid = 1024;         // workgroups a fused launch may have
 
+// floor(a * b / c) for the shares of rows, tiles and workgroups (0 <= a, b; 0 < c; a * b < 2^32, which the host checks
+// for the shapes it accepts).  32-bit on purpose: a 64-bit division is a few hundred instructions on this hardware, and
+// the first one sits in front of every wave's first load.
+__device__ __forceinline__ int mul_div(int a, int b, int c) { return (int)(((unsigned)a * (unsigned)b) / (unsigned)c); }
 __device__ __forceinline__ void counter_add(int* ctr, int v) {
     __hip_atomic_fetch_add(ctr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -584,11 +588,13 @@ __device__ __forceinline__ void finish_refill_row_tile(RowTile<NCH, RPI>& t, con
 // segment, outside the streaming loop (no global store may sit inside it, see RowPark), with the first
 // tile of the next segment already in flight; parked value k (counting from first_index) belongs to the
 // k-th row this wave finished.
+// tiles per flush segment: even, so a segment is a whole number of loop trips
+template <int RPI> constexpr int park_seg_tiles() { return (kParkRows / RPI) & ~1; }
 template <int NCH, int RPI, bool EXACT, bool ROLL = false, class RowOf, class Flush>
 __device__ __forceinline__ void gemv_tiles(const half_t* __restrict__ W, int K, int nrows, int stride_in_tile, int ntiles,
                                            RowOf&& row_of, const half2_t (&x)[NCH][4], int lane, RowTile<NCH, RPI>& pre,
                                            RowPark& park, Flush&& flush) {
-    constexpr int kSegTiles = (kParkRows / RPI) & ~1;   // even, so a segment is a whole number of loop trips
+    constexpr int kSegTiles = park_seg_tiles<RPI>();
     static_assert(kSegTiles >= 2, "tile larger than the park");
     auto valid_rows = [&](int t) {   // only the last tile of a wave can be short
         int v = 0;
@@ -1313,10 +1319,24 @@ __device__ __forceinline__ void down_phases(const StageC& c, int ks, int lane, i
 template <int NCH, int CPD, class DownReady, class OReady>
 __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, StageCShared& sh, bool streamer, int ks,
                                              int o_index, int n_o, int lane, DownReady&& down_ready, OReady&& o_ready) {
-    const int r0 = (int)(((long long)wg * c.nrows) / nwg), r1 = (int)(((long long)(wg + 1) * c.nrows) / nwg);
+    const int r0 = mul_div(wg, c.nrows, nwg), r1 = mul_div(wg + 1, c.nrows, nwg);
     bool first = true;
     for (int b0 = r0; b0 < r1; b0 += kRowBatch) {
         const int b1 = (b0 + kRowBatch < r1) ? b0 + kRowBatch : r1;
+        // what the epilogue of this batch adds to the dot products are inputs of the layer: requested now, so that the
+        // threads that finish the rows do not start a memory round trip after the last barrier
+        float e_b1 = 0.f, e_b2 = 0.f, e_x0 = 0.f, e_x1 = 0.f, e_sa = 0.f, e_sb = 0.f;
+        if ((int)threadIdx.x < b1 - b0) {
+            const int r = b0 + (int)threadIdx.x;
+            if (c.bias1) e_b1 = (float)c.bias1[r];
+            if (c.bias2) e_b2 = (float)c.bias2[r];
+            if (c.base0) e_x0 = (float)c.base0[r];
+            if (c.base1) e_x1 = (float)c.base1[r];
+            if (c.sum_b != nullptr || c.add_sum) {
+                e_sa = (float)c.sum_a[r];
+                if (c.sum_b != nullptr) e_sb = (float)c.sum_b[r];
+            }
+        }
         if (streamer && c.K2 > 0) down_phases<CPD, 0>(c, ks, lane, b0, b1, sh, first, down_ready);
         if (o_index >= 0 && c.K1 > 0) {
             // up to kORows rows of this wave are requested before the attention vector is waited for, so that
@@ -1373,15 +1393,15 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
                 }
             }
             if (c.K1 > 0) v += sh.red_o[t];
-            if (c.bias1) v += (float)c.bias1[r];
-            if (c.bias2) v += (float)c.bias2[r];
-            if (c.base0) v += (float)c.base0[r];
-            if (c.base1) v += (float)c.base1[r];
+            if (c.bias1) v += e_b1;
+            if (c.bias2) v += e_b2;
+            if (c.base0) v += e_x0;
+            if (c.base1) v += e_x1;
             if (c.sum_b != nullptr || c.add_sum) {
                 // the fp16 sum the norm saw; every workgroup is past its norm by now (stage C follows the attention,
                 // which follows all QKV rows), so the sum may overwrite one of its operands
-                float rs = (float)c.sum_a[r];
-                if (c.sum_b != nullptr) rs = (float)(half_t)(rs + (float)c.sum_b[r]);
+                float rs = e_sa;
+                if (c.sum_b != nullptr) rs = (float)(half_t)(rs + e_sb);
                 if (c.sum_out) c.sum_out[r] = (half_t)rs;
                 if (c.add_sum) v += rs;
             }

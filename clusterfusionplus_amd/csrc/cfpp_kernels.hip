@@ -35,7 +35,7 @@ template <int RPI>
 __device__ __forceinline__ RowWalk row_walk(int w, int nw, int lo, int hi) {
     const int units = (hi - lo + RPI - 1) / RPI;
     RowWalk rw;
-    const int u0 = (int)(((long long)w * units) / nw), u1 = (int)(((long long)(w + 1) * units) / nw);
+    const int u0 = mul_div(w, units, nw), u1 = mul_div(w + 1, units, nw);
     rw.first = lo + u0 * RPI; rw.step = RPI; rw.sit = 1; rw.ntiles = u1 - u0;
     rw.end = lo + u1 * RPI < hi ? lo + u1 * RPI : hi;
     return rw;
@@ -91,7 +91,7 @@ __device__ __forceinline__ TileTeam make_team(const LayerParams& p, int pass, in
     const int nteams = (G + kTeamWgs - 1) / kTeamWgs, k = b / kTeamWgs;
     const int wgs = (G - k * kTeamWgs) < kTeamWgs ? (G - k * kTeamWgs) : kTeamWgs;
     const int T = (hi - lo + RPI - 1) / RPI;
-    const int t0 = (int)(((long long)T * k) / nteams), t1 = (int)(((long long)T * (k + 1)) / nteams);
+    const int t0 = mul_div(T, k, nteams), t1 = mul_div(T, k + 1, nteams);
     TileTeam tm;
     tm.counter = p.team + ((size_t)pass * (kMaxGrid / kTeamWgs) + k) * kMailboxInts;
     tm.j = (b - k * kTeamWgs) * kStreamers + wave;
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_up(LayerParams p) {
     const int gw = blockIdx.x * kStreamers + wave, nw = gridDim.x * kStreamers;
     RowPark park{park_mem[wave], 0};
     const int F = p.F;
-    const int first = (int)(((long long)gw * F) / nw), count = (int)(((long long)(gw + 1) * F) / nw) - first;
+    const int first = mul_div(gw, F, nw), count = mul_div(gw + 1, F, nw) - first;
     LnOwn<NCH, kStreamers> own;
     ln_coop_load<NCH, kStreamers, false>(own, norm_spec(p), wave, lane);
     __builtin_amdgcn_sched_barrier(0);   // the norm inputs go out first
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
     const int F = p.F;
     auto share = [&](int g, int& first, int& count) {      // this wave's pairs of phase g
         const int lo = g == 0 ? 0 : up_phase_rows(CPD, g - 1, F), hi = up_phase_rows(CPD, g, F);
-        const int f0 = lo + (int)(((long long)gw * (hi - lo)) / nw), f1 = lo + (int)(((long long)(gw + 1) * (hi - lo)) / nw);
+        const int f0 = lo + mul_div(gw, hi - lo, nw), f1 = lo + mul_div(gw + 1, hi - lo, nw);
         first = f0; count = f1 - f0;
     };
     int first, count;
@@ -819,7 +819,7 @@ __global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
     __shared__ f32x4_t red[NW][64];
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
     const int nblocks = a.R / 16;
-    const int b0 = (int)(((long long)blockIdx.x * nblocks) / gridDim.x), b1 = (int)(((long long)(blockIdx.x + 1) * nblocks) / gridDim.x);
+    const int b0 = mul_div(blockIdx.x, nblocks, gridDim.x), b1 = mul_div(blockIdx.x + 1, nblocks, gridDim.x);
     if (b0 >= b1) return;
     const size_t k0 = (size_t)wave * kChunk;
     unsigned char* mine = stage[wave];
@@ -1003,7 +1003,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gemv_t(GemvT a) {
     const bool in = col < a.O;
     // this wave's rows: slice `slice` of K, quarter `wave` of the slice
     const int part_id = slice * kStreamers + wave, nparts = a.slices * kStreamers;
-    const int k0 = (int)(((long long)part_id * a.K) / nparts), k1 = (int)(((long long)(part_id + 1) * a.K) / nparts);
+    const int k0 = mul_div(part_id, a.K, nparts), k1 = mul_div(part_id + 1, a.K, nparts);
     const half_t* wp = a.W + ((size_t)sec * a.K) * a.O + (in ? col : 0);
     float acc[8];
 #pragma unroll
@@ -2189,10 +2189,13 @@ int launch_lm_head(int H, int vocab, float eps, const void* x, const void* ln_w,
 }
 }  // namespace
 
+// Row shares are worked out in 32 bits on the device (mul_div): wave index x rows must stay below 2^32.  The layer shapes
+// are bounded by check_dims (at most 8192 waves x 16384 rows); the LM head's rows are the vocabulary.
+constexpr int kMaxVocab = 1 << 19;
 int cfpp_neox_lm_head(int32_t hidden, int32_t vocab, float eps, const void* x, const void* ln_w, const void* ln_b,
                       const void* w, float* logits, void* stream) {
     if (!x || !ln_w || !ln_b || !w || !logits) return CFPP_ERR_NULL;
-    if (hidden <= 0 || hidden % 8 || hidden > 8 * kChunk || vocab <= 0) return CFPP_ERR_DIMS;
+    if (hidden <= 0 || hidden % 8 || hidden > 8 * kChunk || vocab <= 0 || vocab > kMaxVocab) return CFPP_ERR_DIMS;
     if (!aligned16(x) || !aligned16(ln_w) || !aligned16(ln_b) || !aligned16(w)) return CFPP_ERR_ALIGN;
     Plan pl{};
     return launch_lm_head(hidden, vocab, eps, x, ln_w, ln_b, w, logits, nullptr, nullptr, grid_for_streaming(pl),
@@ -2277,7 +2280,7 @@ int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out) {
     if (!desc || !out) return CFPP_ERR_NULL;
     int rc = check_dims(&desc->dims);
     if (rc) return rc;
-    if (desc->n_layers <= 0 || desc->vocab <= 0 || desc->cache_rows <= 0) return CFPP_ERR_DIMS;
+    if (desc->n_layers <= 0 || desc->vocab <= 0 || desc->vocab > kMaxVocab || desc->cache_rows <= 0) return CFPP_ERR_DIMS;
     if (!desc->layers || !desc->embed || !desc->final_ln_w || !desc->final_ln_b || !desc->lm_head || !desc->k_caches ||
         !desc->v_caches || !desc->rope_cos || !desc->rope_sin)
         return CFPP_ERR_NULL;

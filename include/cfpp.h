@@ -294,7 +294,7 @@ int cfpp_one_launch_fits(int grid, int compute_units, int blocks_per_cu);
 typedef struct cfpp_neox_stack_desc {
     cfpp_neox_dims dims;
     int32_t n_layers;
-    int32_t vocab;
+    int32_t vocab;                     /* 1 .. 524288 */
     const cfpp_neox_weights* layers;   /* host array [n_layers] of device pointers */
     const void* embed;                 /* [vocab, H] fp16 */
     const void* final_ln_w;            /* [H] fp16 */
@@ -332,7 +332,7 @@ int cfpp_stack_buffers(cfpp_neox_stack* s, float** logits, void** hidden, int32_
 int cfpp_stack_check(cfpp_neox_stack* s, void* stream);
 int cfpp_stack_destroy(cfpp_neox_stack* s);
 
-/* Final LayerNorm + LM-head GEMV: logits[v] = W[v,:] . LN(x) (no bias), fp32 logits.
+/* Final LayerNorm + LM-head GEMV: logits[v] = W[v,:] . LN(x) (no bias), fp32 logits; vocab <= 524288.
  * Counterpart of F.layer_norm + embed_out in the reference loop (tests/benchmark_decode.py:180-187). */
 int cfpp_neox_lm_head(int32_t hidden, int32_t vocab, float eps, const void* x, const void* ln_w,
                       const void* ln_b, const void* w, float* logits, void* stream);

@@ -74,6 +74,10 @@ def test_null_and_mode_errors_launch_nothing(lib):
     assert lib.cfpp_stack_create(None, None) == -1
     assert lib.cfpp_stack_destroy(None) == 0
     assert lib.cfpp_neox_lm_head(4096, 100, ctypes.c_float(1e-5), None, None, None, None, None, None) == -1
+    # a vocabulary beyond what the 32-bit row shares of the kernels cover is refused (-2) before anything is launched
+    buf = ctypes.create_string_buffer(64)
+    ptr = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.cfpp_neox_lm_head(4096, (1 << 19) + 1, ctypes.c_float(1e-5), ptr, ptr, ptr, ptr, ctypes.cast(buf, ctypes.POINTER(ctypes.c_float)), None) == -2
 
 
 def test_one_launch_rule_and_device_status_without_a_gpu(lib):
