@@ -64,6 +64,18 @@ def resource_report(out=None):
     for block in re.split(r"remark: [^\n]*Function Name: ", res.stdout)[1:]:
         name = block.split()[0]
         nice = subprocess.run(["c++filt", name], stdout=subprocess.PIPE, text=True).stdout.strip() or name
+        if nice.startswith("_Z"):
+            # c++filt does not know the _Float16 mangling (DF16_): take the kernel's name and its integer / bool template
+            # arguments out of the mangled name by hand
+            m = re.match(r"_ZN12_GLOBAL__N_1(\d+)", name)
+            if m:
+                n = int(m.group(1))
+                base = name[m.end():m.end() + n]
+                targs = re.match(r"I((?:L[ib]\d+E)+)E", name[m.end() + n:])
+                if targs:
+                    vals = [v if k == "i" else ("true" if v == "1" else "false") for k, v in re.findall(r"L([ib])(\d+)E", targs.group(1))]
+                    base += "<" + ", ".join(vals) + ">"
+                nice = base
         nice = nice.replace("(anonymous namespace)::", "").replace("void ", "")
         nice = re.sub(r"\(.*\)$", "", nice)
 
