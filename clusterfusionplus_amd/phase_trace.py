@@ -41,12 +41,14 @@ def synthetic_decoder(cfg, rows, device):
 def main():
     from . import PYTHIA_2B8, PYTHIA_6B9, debug_set_trace
     ap = argparse.ArgumentParser(description=__doc__)
-    ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8"])
+    ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8", "llama2_7b_attention"])
     ap.add_argument("--ctx", type=int, default=2048)
     ap.add_argument("--raw", help="also save the raw timestamps of every layer ([layer][workgroup][wave][slot]) as .npy")
     a = ap.parse_args()
-    cfg = PYTHIA_6B9 if a.model == "pythia_6b9" else PYTHIA_2B8
     dev = "cuda:0"
+    if a.model == "llama2_7b_attention":
+        return llama_attention(a, dev)
+    cfg = PYTHIA_6B9 if a.model == "pythia_6b9" else PYTHIA_2B8
     dec = synthetic_decoder(cfg, a.ctx + 64, dev)
     dec.set_state(11, a.ctx)
     for _ in range(3):
@@ -74,8 +76,44 @@ def main():
     debug_set_trace(None)
     if a.raw:
         np.save(a.raw, np.stack(per_layer))
+    report(per_layer[2:])
+    return 0
+
+
+def llama_attention(a, dev):
+    """The LLaMA-2-7B attention block (fused add + RMSNorm, QKV, attention, O: the fused kernel without an MLP) over eight
+    weight sets in turn."""
+    import clusterfusion as cf
+    from . import debug_set_trace
+    H, heads, S = 4096, 32, a.ctx
+    torch.manual_seed(0)
+
+    def rn(shape, std, mean=0.0):
+        return torch.empty(shape, dtype=torch.float16, device=dev).normal_(mean, std)
+    sets = [(rn((3 * H, H), 0.02), rn((H, H), 0.02), rn((S + 1, H), 1.0), rn((S + 1, H), 1.0), rn((H,), 0.02, 1.0)) for _ in range(8)]
+    x, res = rn((1, H), 1.0), rn((1, H), 1.0)
+    ang = torch.rand(1, 64, device=dev) * 6.28
+    cos, sin = torch.cat([ang.cos(), ang.cos()], -1).float(), torch.cat([ang.sin(), ang.sin()], -1).float()
+    tr = torch.zeros(1024 * 16 * 16, dtype=torch.int64, device=dev)
+    debug_set_trace(tr)
+    per_launch = []
+    for it in range(24):
+        wq, wo, k, v, rms = sets[it % 8]
+        tr.zero_()
+        cf.llama_decoder_layer_sglang(x, res.clone(), wq, wo, k[:S], v[:S], rms, 1e-5, cos, sin, heads)
+        torch.cuda.synchronize()
+        per_launch.append(tr.cpu().numpy().reshape(1024, 16, 16)[:256, :8].astype(np.float64))
+    debug_set_trace(None)
+    if a.raw:
+        np.save(a.raw, np.stack(per_launch))
+    print(f"llama2_7b attention block, context {S}: phase stamps of the fused kernel (profiling build)")
+    report(per_launch[8:])
+    return 0
+
+
+def report(launches):
     rows = {}
-    for raw in per_layer[2:]:
+    for raw in launches:
         t0 = raw[:, :, 0][raw[:, :, 0] > 0].min()
         us = (raw - t0) / 100.0
         for slot, label, who in SLOTS:
@@ -88,7 +126,6 @@ def main():
         if (slot, who) in rows:
             m = np.median(np.array(rows[(slot, who)]), axis=0)
             print(f"{label + ' [' + who + ' waves]':84s} {m[0]:7.2f} {m[1]:7.2f} {m[2]:7.2f} {m[3]:7.2f}")
-    return 0
 
 
 if __name__ == "__main__":
