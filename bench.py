@@ -132,14 +132,18 @@ def drop_in_loop(model, cfg, dec, ctx, tokens=24, warm=4):
     seq = torch.tensor([ctx], dtype=torch.int32, device=dev)
     tok = torch.tensor([11], dtype=torch.int64, device=dev)
 
-    def one_token():
+    def one_token(library_head=False):
         h = t["embed"].index_select(0, tok)
         for l, w in enumerate(t["layers"]):
             h, _, _ = step(base + l, h, w["ln_w"], w["ln_b"], w["b_qkv"], w["b_o"], dec.cos, dec.sin, t["k_caches"][l], t["v_caches"][l],
                            w["post_ln_w"], w["post_ln_b"], w["b_up"], w["b_down"], seq)
-        h = torch.nn.functional.layer_norm(h, (H,), t["final_ln_w"], t["final_ln_b"], eps=cfg.eps)
-        logits = torch.matmul(h, t["lm_head"].t())
-        tok.copy_(torch.argmax(logits, dim=-1))
+        if library_head:
+            # final LayerNorm + LM head in the library (one launch), argmax in torch
+            logits = cf.lm_head(h, t["final_ln_w"], t["final_ln_b"], t["lm_head"], cfg.eps)
+        else:
+            h = torch.nn.functional.layer_norm(h, (H,), t["final_ln_w"], t["final_ln_b"], eps=cfg.eps)
+            logits = torch.matmul(h, t["lm_head"].t())
+        tok.copy_(torch.argmax(logits, dim=-1).reshape(1))
         seq.add_(1)
 
     side = torch.cuda.Stream()
@@ -157,26 +161,36 @@ def drop_in_loop(model, cfg, dec, ctx, tokens=24, warm=4):
     torch.cuda.synchronize()
     eager = e0.elapsed_time(e1) / 4
     eager_wall = (time.perf_counter() - t0) * 1e3 / 4
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        one_token()
-    seq.fill_(ctx)
-    for _ in range(warm):
-        graph.replay()
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(tokens):
-        graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    tpot = e0.elapsed_time(e1) / tokens
-    assert int(seq.item()) == ctx + warm + tokens
+    def captured(library_head):
+        with torch.cuda.stream(side):
+            one_token(library_head)      # warm-up outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            one_token(library_head)
+        seq.fill_(ctx)
+        for _ in range(warm):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(tokens):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        assert int(seq.item()) == ctx + warm + tokens
+        return e0.elapsed_time(e1) / tokens
+    tpot = captured(False)
+    tpot_lib = captured(True)
     for l in range(L):
         destroy(base + l)                # raises if a step of the context failed on the device
     sb = step_bytes(cfg, ctx + warm + tokens // 2)
     return {"workload": f"{model}: per-layer contexts, {L} x {model}_graph_decode_step per token with a device current_seq_len, final "
                         "LayerNorm + LM head + argmax in torch, captured once with torch.cuda.graph and replayed",
             "context": ctx, "tokens": tokens, "tpot_ms": round(tpot, 4), "frac_of_peak": round(sb / (tpot * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "library_lm_head_tpot_ms": round(tpot_lib, 4),
+            "library_lm_head_frac_of_peak": round(sb / (tpot_lib * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "library_lm_head_note": "same loop with the final LayerNorm + LM head in the library (lm_head op), argmax in torch",
             "eager_python_loop_tpot_ms": round(max(eager, eager_wall), 4)}
 
 
@@ -224,6 +238,60 @@ def cpu_baseline(cfg, S, budget_s=12.0):
         "sample": f"{impl}, fp32 eager, 1 layer at S={S} x {len(times)} runs (median {layer_ms:.2f} ms) scaled x{cfg.n_layers}"
                   f" + fp32 LM head matvec ({lm_ms:.2f} ms)",
     }
+
+
+def bench_single_layer(model, S, steps=160, warmup=16, nset=8):
+    """One decoder layer through the drop-in ops (`<model>_decoder_layer` and `<model>_decoder_layer_split`), batch-1
+    decode at context S, replayed from a captured graph that cycles through `nset` weight and cache sets (more than the
+    256 MB Infinity Cache holds), so that every launch reads HBM-cold data.  Returns {mode: us per layer}."""
+    import torch
+    import clusterfusion as cf
+    import clusterfusionplus_amd as pkg
+    dev = "cuda:0"
+    cfg = pkg.PYTHIA_2B8 if model == "pythia_2b8" else pkg.PYTHIA_6B9
+    H, F = cfg.hidden, cfg.ffn
+    torch.manual_seed(5)
+
+    def rn(shape, std, mean=0.0):
+        return torch.empty(shape, dtype=torch.float16, device=dev).normal_(mean, std)
+    sets = []
+    for _ in range(nset):
+        sets.append([rn((3 * H, H), 0.02), rn((3 * H,), 0.01), rn((H, H), 0.02), rn((H,), 0.01), rn((S + 1, H), 1.0), rn((S + 1, H), 1.0),
+                     rn((H,), 0.02, 1.0), rn((H,), 0.01), None, None, rn((H,), 0.02, 1.0), rn((H,), 0.01), rn((F, H), 0.02), rn((F,), 0.01),
+                     rn((H, F), 0.02), rn((H,), 0.01)])
+    x = rn((1, H), 1.0)
+    cos_t, sin_t = pkg.rope_tables(S + 1, cfg.rotary_dim, cfg.rope_base, device=dev)
+    cos, sin = cos_t[S:S + 1].contiguous(), sin_t[S:S + 1].contiguous()
+    for a in sets:
+        a[8], a[9] = cos, sin
+    out = {}
+    for mode, name in (("fused", f"{model}_decoder_layer"), ("split", f"{model}_decoder_layer_split")):
+        op = getattr(cf, name)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for a in sets:
+                op(x, *a, S)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            keep = [op(x, *a, S) for a in sets]
+        for _ in range(max(1, warmup // nset)):
+            graph.replay()
+        torch.cuda.synchronize()
+        reps = max(1, steps // nset)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        out[mode] = e0.elapsed_time(e1) * 1e3 / (reps * nset)
+        del graph, keep
+    if cf.device_status() != 0:
+        raise RuntimeError("a layer launch raised a device-side failure flag")
+    return out
 
 
 def bench_llama_layer(args, emit=True):
@@ -394,6 +462,24 @@ def other_workloads(pkg, dev, args):
         a.ctx, a.batch, a.steps, a.warmup = 1024, 16, 60, 12
         return brief(bench_llama_batch(a, emit=False))
 
+    def single_layer(model, S, config_no):
+        cfg = pkg.PYTHIA_2B8 if model == "pythia_2b8" else pkg.PYTHIA_6B9
+        us = bench_single_layer(model, S)
+        lb = layer_bytes(cfg, S)
+        res = {"workload": f"BASELINE config {config_no}: one {model} decoder layer, batch 1, context {S}, graph replay over 8 weight "
+                           "and cache sets (HBM-cold), fused and split ops", "metric": "layer_latency_us", "unit": "us/layer",
+               "bytes": lb, "roofline_us": round(lb / (HBM_PEAK_GBPS * 1e9) * 1e6, 2)}
+        for mode in ("fused", "split"):
+            res[f"{mode}_us"] = round(us[mode], 2)
+            res[f"{mode}_frac_of_peak"] = round(lb / (us[mode] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
+        res["value"] = res["fused_us"]
+        res["frac_of_peak"] = res["fused_frac_of_peak"]
+        return res
+
+    attempt("pythia_2b8 single layer (config 1)", lambda: single_layer("pythia_2b8", 512, 1))
+    torch.cuda.empty_cache()
+    attempt("pythia_6b9 single layer (config 3)", lambda: single_layer("pythia_6b9", 2048, 3))
+    torch.cuda.empty_cache()
     attempt("pythia_2b8 full stack", stack_2b8)
     torch.cuda.empty_cache()
     attempt("llama2_7b decoder layer", llama_layer)
@@ -511,6 +597,23 @@ def main():
                                 "hbm_gbps": result["step"]["hbm_gbps"], "frac_of_peak": result["step"]["frac_of_peak"]}] + \
                 context_sweep(dec, cfg, stream, sweep_ctx)
         result["sweep"].sort(key=lambda r: r["context"])
+        try:
+            # the same model through the per-stage launches (CFPP_MODE_SPLIT), sharing the weights and caches
+            sdec = pkg.NeoxDecoder(cfg, dec.tensors["layers"], dec.tensors["embed"], dec.tensors["final_ln_w"], dec.tensors["final_ln_b"],
+                                   dec.tensors["lm_head"], dec.tensors["k_caches"], dec.tensors["v_caches"], mode="split")
+            with torch.cuda.stream(stream):
+                st = time_tokens(sdec, stream, args.ctx, 32, 6)
+            sdec.check()
+            ssb = step_bytes(cfg, args.ctx + 6 + 16)
+            result["split_mode"] = {"workload": f"{args.model} full stack, split mode (one launch per stage instead of one per layer), "
+                                                f"hipGraph replay, context {args.ctx}", "context": args.ctx, "tokens": 32,
+                                    "tpot_ms": round(st, 4), "bytes": ssb, "hbm_gbps": round(ssb / (st * 1e-3) / 1e9, 1),
+                                    "frac_of_peak": round(ssb / (st * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+            log(f"[split] context {args.ctx}: {st:.4f} ms/token = {result['split_mode']['frac_of_peak'] * 100:.1f} % of peak")
+            del sdec
+        except Exception as e:     # noqa: BLE001
+            log(f"[split_mode] failed: {type(e).__name__}: {e}")
+            result["split_mode"] = {"error": f"{type(e).__name__}: {e}"}
         try:
             result["drop_in_loop"] = drop_in_loop(args.model, cfg, dec, args.ctx)
             result["drop_in_loop"]["neox_decoder_tpot_ms"] = round(tpot, 4)

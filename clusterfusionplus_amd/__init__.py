@@ -36,7 +36,7 @@ if not _missing:
     globals().update({n: getattr(_native, n) for n in __all__})
 
     from .model import (NeoxConfig, PYTHIA_2B8, PYTHIA_6B9, NeoxDecoder, layer_tensor_order, rope_tables,  # noqa: E402
-                        layer_tensors_from_hf, kv_cache_from_hf)
+                        layer_tensors_from_hf, kv_cache_from_hf, config_from_hf, stack_tensors_from_hf)
 
     __all__ += ["NeoxConfig", "PYTHIA_2B8", "PYTHIA_6B9", "NeoxDecoder", "layer_tensor_order", "rope_tables",
-                "layer_tensors_from_hf", "kv_cache_from_hf"]
+                "layer_tensors_from_hf", "kv_cache_from_hf", "config_from_hf", "stack_tensors_from_hf"]

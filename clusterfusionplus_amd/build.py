@@ -26,6 +26,9 @@ HIPCC_FLAGS = [
     # packed-fp32 arithmetic stays off in device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # one name for the product build and for profiling builds kept elsewhere: a process that has loaded either one
+    # resolves the binding's dependency on "libcfpp.so" to it
+    "-Wl,-soname,libcfpp.so",
 ]
 
 
@@ -41,7 +44,10 @@ def _run(cmd):
 
 def build_lib(trace: bool = False, out: str = LIB):
     """libcfpp.so.  `trace`: a profiling build (-DCFPP_TRACE) whose fused kernel stores phase timestamps for
-    `python -m clusterfusionplus_amd.phase_trace`; it is slower by the stores and is never the default."""
+    `python clusterfusionplus_amd/phase_trace.py --trace-lib PATH`; it is slower by the stores, is written to a path
+    of its own and never takes the place of the product library."""
+    if trace and os.path.abspath(out) == os.path.abspath(LIB):
+        raise ValueError("a profiling build must not overwrite the product library; give it a path of its own")
     hipcc = os.path.join(ROCM, "bin", "hipcc")
     extra = ["-DCFPP_TRACE"] if trace else []
     _run([hipcc, *HIPCC_FLAGS, *extra, f"-I{INCLUDE}", f"-I{CSRC}", os.path.join(CSRC, "cfpp_kernels.hip"), "-o", out])
@@ -119,7 +125,8 @@ def build_all():
 if __name__ == "__main__":
     import argparse
     ap = argparse.ArgumentParser(description=__doc__)
-    ap.add_argument("--trace-lib", metavar="PATH", help="only build a profiling variant of libcfpp.so (-DCFPP_TRACE) at PATH")
+    ap.add_argument("--trace-lib", metavar="PATH",
+                    help="only build a profiling variant of the HIP library (-DCFPP_TRACE) at PATH (not the product library's path)")
     ap.add_argument("--resource-report", action="store_true",
                     help="only print registers, scratch, LDS and occupancy of every kernel (compiler remarks)")
     a = ap.parse_args()

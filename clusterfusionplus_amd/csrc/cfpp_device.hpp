@@ -78,6 +78,7 @@ struct LayerParams {
                             // 1 = they hold rot/2 entries, the angles of the pairs, and dims d and d + rot/2 share entry d
     int seq_len;
     const int* d_seq_len;
+    int seq_cap;        // largest sequence length the launch geometry was sized for (a device-side length beyond it is refused)
     int max_split;      // cap on the KV splits per head (<= kMaxSplit)
     const int* kv_rows;     // paged caches: cache row r of this sequence lives in row kv_rows[r] of k_cache / v_cache (null: r itself)
     const int* tag_src;     // launch tags from a counter the caller advances between launches (null: from kBarGen)
@@ -254,12 +255,13 @@ __device__ __forceinline__ void counter_add(int* ctr, int v) {
 __device__ __forceinline__ int counter_peek(const int* ctr) {
     return __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// Failure flags go to the workspace's status word and, when the launch has one, to a word in pinned host memory
-// (a plain system-scope store of the flag: the host only asks whether it is non-zero).
+// Failure flags go to the workspace's status word and, when the launch has one, to pinned host memory: one word
+// per flag (host[0] for kStatusSpin, host[1] for kStatusSeq), written with a plain system-scope store, so that two
+// different flags never overwrite each other and no read-modify-write has to cross the bus.
 struct StatusSink { int* dev; int* host; };
 __device__ __forceinline__ void raise_status(const StatusSink& s, int flag) {
     __hip_atomic_fetch_or(s.dev, flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (s.host != nullptr) __hip_atomic_store(s.host, flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (s.host != nullptr) __hip_atomic_store(s.host + (flag == kStatusSpin ? 0 : 1), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 // Arrivals are counted hierarchically, because a thousand waves adding to one address serialise at the
 // memory side (tens of nanoseconds each) and every one of them waits for its return value: first in LDS
@@ -326,12 +328,14 @@ __device__ __forceinline__ StatusSink status_sink(const LayerParams& p) { return
 // The number of valid cache rows S of this step.  A host-side length may equal the cache rows (the append is then
 // skipped, k_new / v_new are still returned).  A device-side length, or RoPE tables indexed by the position
 // (rope_stride > 0, one table row per cache row), need S < cache_rows: the step reads table row S and appends cache
-// row S.  Anything else raises kStatusSeq; the step then runs on a clamped length without appending, so that no
-// access leaves the caches or the tables, and its results mean nothing.
+// row S.  A device-side length must also stay within seq_cap, the bound the host sized the launches for (the grid of the
+// attention items in split mode).  Anything else raises kStatusSeq; the step then runs on a clamped length without
+// appending, so that no access leaves the caches or the tables, and its results mean nothing.
 struct SeqLen { int S; bool ok; };
 __device__ __forceinline__ SeqLen load_seq_len(const LayerParams& p) {
     int S = p.d_seq_len ? *p.d_seq_len : p.seq_len;
-    const int limit = (p.d_seq_len != nullptr || p.rope_stride > 0) ? p.cache_rows - 1 : p.cache_rows;
+    int limit = (p.d_seq_len != nullptr || p.rope_stride > 0) ? p.cache_rows - 1 : p.cache_rows;
+    if (p.d_seq_len != nullptr && p.seq_cap < limit) limit = p.seq_cap;
     const bool ok = S >= 0 && S <= limit;
     if (!ok) {
         if (threadIdx.x == 0 && blockIdx.x == 0) raise_status(status_sink(p), kStatusSeq);

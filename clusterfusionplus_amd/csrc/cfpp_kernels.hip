@@ -125,30 +125,74 @@ __device__ __forceinline__ void up_team_rows(const LayerParams& p, const half2_t
 }
 
 // ---- split mode: one launch per stage ----------------------------------------------------------
-// Four waves per workgroup everywhere: one per SIMD.  A second wave on a SIMD gets far less of the
-// memory pipeline than the first while both stream, so extra streaming waves only add imbalance.
-template <int NCH, bool EX>
-__global__ __launch_bounds__(kStreamers * 64) void k_stage_a(LayerParams p) {
-    __shared__ float park_mem[kStreamers][kParkRows];
+// Three launches; no workgroup waits for another inside any of them (the kernel boundary is the barrier), so this mode
+// runs wherever the one-launch kernel cannot be guaranteed its co-residency (reference
+// include/5090/pythia_2b8/pythia_kernel_dispatch_split.cu:158-214 splits at the same places, QKV | attention | MLP, but
+// runs its stages strictly one after the other):
+//   k_stage_qkv   LayerNorm + QKV rows, NW waves per workgroup (eight when that leaves every wave three tiles);
+//   k_stage_mid   eight waves per workgroup: four stream the MLP-up rows (they depend on the layer input only), four
+//                 run the (head, split) attention items - a chain of dependent round trips that would otherwise be a
+//                 launch of its own with nothing to hide behind;
+//   k_stage_c     O projection on four waves beside the MLP-down rows on the other four, residual.
+template <int NCH, int NW, bool EX>
+__global__ __launch_bounds__(NW * 64) void k_stage_qkv(LayerParams p) {
+    __shared__ float park_mem[NW][kParkRows];
     __shared__ LnShared<NCH> lns;
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
-    const int gw = blockIdx.x * kStreamers + wave, nw = gridDim.x * kStreamers;
+    const int gw = blockIdx.x * NW + wave, nw = gridDim.x * NW;
     RowPark park{park_mem[wave], 0};
     const RowWalk qw = row_walk<StageARpi<NCH>::value>(gw, nw, 0, 3 * p.H);
-    LnOwn<NCH, kStreamers> own;
-    ln_coop_load<NCH, kStreamers, true>(own, norm_spec(p), wave, lane);
+    LnOwn<NCH, NW> own;
+    ln_coop_load<NCH, NW, false>(own, norm_spec(p), wave, lane);
     __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
     RowTile<NCH, StageARpi<NCH>::value> t0;
     qkv_prefetch<NCH, EX>(p, qw, lane, t0);
-    ln_coop_finish<NCH, kStreamers, true>(own, norm_spec(p), lns, wave, lane);
+    ln_coop_finish<NCH, NW, false>(own, norm_spec(p), lns, wave, lane);
     half2_t xr[NCH][4];
     ln_fetch<NCH>(lns, 0, lane, xr);
     qkv_rows<NCH, EX>(p, xr, qw, lane, t0, park);
-    const RowWalk uw = row_walk<kUpRpi>(gw, nw, 0, p.F);
+}
+
+// MLP-up rows on the streaming waves, attention items on the other four; wave hw of workgroup b takes the items
+// b + hw G, + 4 G, ... (any number of items: nothing here waits for another workgroup).
+template <int NCH, bool EX>
+__global__ __launch_bounds__(2 * kStreamers * 64) void k_stage_mid(LayerParams p) {
+    __shared__ float park_mem[kStreamers][kParkRows];
+    __shared__ LnShared<NCH> lns;
+    constexpr int NW = 2 * kStreamers;
+    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int G = gridDim.x, b = blockIdx.x;
+    const int hw = wave - kStreamers;
+    const SeqLen sl = load_seq_len(p);
+    const int nsplit = effective_split(p, sl.S), per_head = items_per_head(nsplit);
+    const int nitems = p.heads * per_head;
+    AttnItem it;
+    int item = b + hw * G;
+    // an attention wave's first item is requested before the LayerNorm (it needs none of it) ...
+    if (hw >= 0 && item < nitems) attn_prefetch(p, it, item / per_head, item % per_head, nsplit, sl, lane);
+    // ... the post-attention LayerNorm of the input row, by all eight waves (slot 0 holds it: only one row is needed here)
+    NormSpec ns = norm_spec(p);
+    ns.w1 = p.ln2_w; ns.b1 = p.ln2_b;
+    LnOwn<NCH, NW> own;
+    ln_coop_load<NCH, NW, false>(own, ns, wave, lane);
+    __builtin_amdgcn_sched_barrier(0);
     RowTile<NCH, kUpRpi> u0;
-    up_prefetch<NCH, EX>(p, uw, lane, u0);
-    ln_fetch<NCH>(lns, 1, lane, xr);
-    up_rows<NCH, EX>(p, xr, uw, lane, u0, park);
+    const RowWalk uw = row_walk<kUpRpi>(b * kStreamers + (hw < 0 ? wave : 0), G * kStreamers, 0, hw < 0 ? p.F : 0);
+    if (hw < 0) up_prefetch<NCH, EX>(p, uw, lane, u0);
+    ln_coop_finish<NCH, NW, false>(own, ns, lns, wave, lane);
+    if (hw < 0) {
+        RowPark park{park_mem[wave], 0};
+        half2_t xr[NCH][4];
+        ln_fetch<NCH>(lns, 0, lane, xr);
+        up_rows<NCH, EX>(p, xr, uw, lane, u0, park);
+    } else {
+        __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
+        while (item < nitems) {
+            attention_item(p, it, lane, 0, 0);
+            item += kStreamers * G;
+            if (item < nitems) attn_prefetch(p, it, item / per_head, item % per_head, nsplit, sl, lane);
+        }
+    }
 }
 
 // Norm + gated MLP-up (SwiGLU): inter[r] = silu(Wg[r] . n) * (Wu[r] . n), n = norm(x), with p.w_up = [Wg; Wu] ([2F, H]).
@@ -256,6 +300,17 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
     const int wave = first_lane(threadIdx.x >> 6);
     const StageC c = make_stage_c(p);
     stage_c_rows<NCH, CPD>(c, blockIdx.x, gridDim.x, sh, true, wave, wave, kStreamers, threadIdx.x & 63, [](int) {}, [] {});
+}
+// The same with eight waves, shared out as in the one-launch kernel: MLP-down rows on four waves, the O projection on the
+// other four (all eight when there is no MLP-down pass).  Which wave computes a row does not change its value.
+template <int NCH, int CPD>
+__global__ __launch_bounds__(2 * kStreamers * 64) void k_stage_c8(LayerParams p) {
+    __shared__ StageCShared sh;
+    const int wave = first_lane(threadIdx.x >> 6);
+    const StageC c = make_stage_c(p);
+    const bool streamer = wave < kStreamers, all_o = c.K2 == 0;
+    stage_c_rows<NCH, CPD>(c, blockIdx.x, gridDim.x, sh, streamer, wave, all_o ? wave : (streamer ? -1 : wave - kStreamers),
+                           all_o ? 2 * kStreamers : kStreamers, threadIdx.x & 63, [](int) {}, [] {});
 }
 
 // ---- fused mode: one persistent launch ---------------------------------------------------------
@@ -1159,11 +1214,10 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_attn(LayerParams p, B
 struct DeviceInfo {
     int cus = 0;
     bool ok = false;
-    int* host_status = nullptr;        // one word of pinned host memory: device-side failure flags land here as well
-    int* host_status_dev = nullptr;    // the device's address of that word
+    int* host_status = nullptr;        // a line of pinned host memory: device-side failure flags land here as well, one word per flag
+    int* host_status_dev = nullptr;    // the device's address of that line
     std::map<const void*, int> blocks_per_cu;   // occupancy of the one-launch kernels, by kernel
     void* static_scratch = nullptr;    // address of this device's copy of the file-scope scratch array
-    unsigned long long static_key = 0; // geometry of the last call that used it (0: never used)
 };
 std::mutex g_device_mu;
 
@@ -1174,69 +1228,70 @@ std::mutex g_device_mu;
 constexpr size_t kStaticScratchBytes = 1280u << 10;      // 1.25 MiB: a Pythia-6.9B layer needs 1.19 MiB
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
-// set while an entry point that must not allocate runs on this thread: the per-device set-up then skips the pinned
-// status word (it is added by the next ordinary call)
+// set while an entry point that must not allocate runs on this thread: the per-device set-up then does not create the
+// pinned status line (that entry point refuses to run without it, see cfpp_neox_layer_decode_static)
 thread_local bool tl_no_alloc = false;
 
+// The per-device record, set up under the lock on first use (compute units; the pinned status line unless the calling
+// entry point must not allocate).  Every field is written under g_device_mu and never changes once set.
 DeviceInfo& device_info() {
     static DeviceInfo info[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     DeviceInfo& d = info[dev];
+    std::lock_guard<std::mutex> lock(g_device_mu);
     if (!d.ok) {
-        std::lock_guard<std::mutex> lock(g_device_mu);
-        if (!d.ok) {
-            hipDeviceProp_t prop;
-            if (hipGetDeviceProperties(&prop, dev) == hipSuccess) {
-                d.cus = prop.multiProcessorCount;
-                d.ok = true;
-            }
-            (void)hipGetLastError();
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) == hipSuccess) {
+            d.cus = prop.multiProcessorCount;
+            d.ok = true;
         }
+        (void)hipGetLastError();
     }
     if (d.ok && d.host_status == nullptr && !tl_no_alloc) {
-        std::lock_guard<std::mutex> lock(g_device_mu);
-        if (d.host_status == nullptr) {
-            void* h = nullptr;
-            if (hipHostMalloc(&h, 64, hipHostMallocMapped) == hipSuccess && h != nullptr) {
-                *reinterpret_cast<volatile int*>(h) = 0;
-                void* dp = nullptr;
-                if (hipHostGetDevicePointer(&dp, h, 0) == hipSuccess && dp != nullptr) {
-                    d.host_status_dev = reinterpret_cast<int*>(dp);
-                    d.host_status = reinterpret_cast<int*>(h);
-                } else {
-                    (void)hipHostFree(h);
-                }
+        void* h = nullptr;
+        if (hipHostMalloc(&h, 64, hipHostMallocMapped) == hipSuccess && h != nullptr) {
+            std::memset(h, 0, 64);
+            void* dp = nullptr;
+            if (hipHostGetDevicePointer(&dp, h, 0) == hipSuccess && dp != nullptr) {
+                d.host_status_dev = reinterpret_cast<int*>(dp);
+                d.host_status = reinterpret_cast<int*>(h);
+            } else {
+                (void)hipHostFree(h);
             }
-            (void)hipGetLastError();
         }
+        (void)hipGetLastError();
     }
     return d;
+}
+
+// The failure flags the kernels have stored in the pinned status line of a device (one word per flag), as a bit mask.
+int host_status_flags(const DeviceInfo& di, bool clear) {
+    if (!di.host_status) return 0;
+    volatile int* w = reinterpret_cast<volatile int*>(di.host_status);
+    const int flags = (w[0] ? kStatusSpin : 0) | (w[1] ? kStatusSeq : 0);
+    if (clear) { w[0] = 0; w[1] = 0; }
+    return flags;
 }
 
 // The address of the current device's copy of `scratch`, looked up on first use per device.
 int static_scratch_address(void** out) {
     DeviceInfo& di = device_info();
     if (!di.ok) return (int)hipErrorNoDevice;
+    std::lock_guard<std::mutex> lock(g_device_mu);
     if (di.static_scratch == nullptr) {
-        std::lock_guard<std::mutex> lock(g_device_mu);
-        if (di.static_scratch == nullptr) {
-            void* ptr = nullptr;
-            const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-            if (e != hipSuccess) return (int)e;
-            if (ptr == nullptr || (reinterpret_cast<uintptr_t>(ptr) & 255u)) return (int)hipErrorInvalidSymbol;
-            di.static_scratch = ptr;
-        }
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (ptr == nullptr || (reinterpret_cast<uintptr_t>(ptr) & 255u)) return (int)hipErrorInvalidSymbol;
+        di.static_scratch = ptr;
     }
     *out = di.static_scratch;
     return CFPP_OK;
 }
 
 // non-zero: some launch on this device has raised a failure flag since the word was last cleared
-int pending_device_failure() {
-    DeviceInfo& di = device_info();
-    return di.host_status ? *reinterpret_cast<volatile int*>(di.host_status) : 0;
-}
+int pending_device_failure() { return host_status_flags(device_info(), false); }
 #define CFPP_REFUSE_AFTER_FAILURE()                          \
     do {                                                     \
         if (pending_device_failure()) return CFPP_ERR_DEVICE; \
@@ -1314,14 +1369,31 @@ thread_local KernelEvents* tl_kernel_events = nullptr;
 
 // ---- template dispatch ---------------------------------------------------------------------------
 template <int NCH>
-int launch_stage_a_t(const LayerParams& p, int grid, hipStream_t st) {
-    if (p.H == NCH * kChunk) hipLaunchKernelGGL((k_stage_a<NCH, true>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
-    else hipLaunchKernelGGL((k_stage_a<NCH, false>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
+int launch_stage_qkv_t(const LayerParams& p, int grid, hipStream_t st) {
+    // eight waves per workgroup when every wave still gets three tiles (twice the loads in flight), else four
+    constexpr int RPIA = StageARpi<NCH>::value;
+    const bool wide = (3 * p.H + RPIA - 1) / RPIA >= 3 * grid * 2 * kStreamers;
+    const bool ex = p.H == NCH * kChunk;
+    if (wide) {
+        if (ex) hipLaunchKernelGGL((k_stage_qkv<NCH, 2 * kStreamers, true>), dim3(grid), dim3(2 * kStreamers * 64), 0, st, p);
+        else hipLaunchKernelGGL((k_stage_qkv<NCH, 2 * kStreamers, false>), dim3(grid), dim3(2 * kStreamers * 64), 0, st, p);
+    } else {
+        if (ex) hipLaunchKernelGGL((k_stage_qkv<NCH, kStreamers, true>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
+        else hipLaunchKernelGGL((k_stage_qkv<NCH, kStreamers, false>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
+    }
     return launch_check();
 }
+template <int NCH>
+int launch_stage_mid_t(const LayerParams& p, int grid, hipStream_t st) {
+    if (p.H == NCH * kChunk) hipLaunchKernelGGL((k_stage_mid<NCH, true>), dim3(grid), dim3(2 * kStreamers * 64), 0, st, p);
+    else hipLaunchKernelGGL((k_stage_mid<NCH, false>), dim3(grid), dim3(2 * kStreamers * 64), 0, st, p);
+    return launch_check();
+}
+// stage C: eight waves when the O projection is part of it, four for the MLP-down rows alone
 template <int NCH, int CPD>
 int launch_stage_c_t(const LayerParams& p, int grid, hipStream_t st) {
-    hipLaunchKernelGGL((k_stage_c<NCH, CPD>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
+    if (p.c_use_o) hipLaunchKernelGGL((k_stage_c8<NCH, CPD>), dim3(grid), dim3(2 * kStreamers * 64), 0, st, p);
+    else hipLaunchKernelGGL((k_stage_c<NCH, CPD>), dim3(grid), dim3(kStreamers * 64), 0, st, p);
     return launch_check();
 }
 // The one-launch kernels wait for each other's workgroups inside the launch, so every workgroup of the grid has to
@@ -1332,7 +1404,7 @@ int launch_stage_c_t(const LayerParams& p, int grid, hipStream_t st) {
 // one-launch kernel starts can keep some of its workgroups waiting; the bounded waits then expire, the failure flag
 // is raised and the next call on the device reports CFPP_ERR_DEVICE.
 bool one_launch_fits(const void* fn, int block_threads, int grid) {
-    DeviceInfo& di = device_info();
+    DeviceInfo& di = device_info();     // (takes and releases the lock itself)
     int per_cu = 0;
     {
         std::lock_guard<std::mutex> lock(g_device_mu);
@@ -1374,15 +1446,24 @@ int launch_fused_t(const LayerParams& p, int grid, hipStream_t st) {
 template <int NCH, int CPD>
 bool fused_fits_t(const LayerParams& p, int grid) { return one_launch_fits(fused_fn<NCH, CPD>(p, grid), 2 * kStreamers * 64, grid); }
 
-#define CFPP_NCH_CASES(X) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8)
+// hidden chunks that occur in CFPP_SHAPE_CASES below
+#define CFPP_NCH_CASES(X) X(1) X(2) X(4) X(5) X(8)
 // (hidden chunks, MLP-down chunks per streaming wave).  The Pythia family has ffn = 4 hidden, so both
 // numbers coincide: 512 -> (1,1), 768/1024 -> (2,2), 2048 -> (4,4), 2560 -> (5,5), 4096 -> (8,8);
 // (8,6) is hidden 4096 with ffn 11008
 #define CFPP_SHAPE_CASES(X) X(1, 1) X(2, 2) X(4, 4) X(5, 5) X(8, 8) X(8, 6)
 
-int launch_stage_a(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
+int launch_stage_qkv(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
     switch (pl.nch) {
-#define X(n) case n: return launch_stage_a_t<n>(p, grid, st);
+#define X(n) case n: return launch_stage_qkv_t<n>(p, grid, st);
+        CFPP_NCH_CASES(X)
+#undef X
+    }
+    return CFPP_ERR_DIMS;
+}
+int launch_stage_mid(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
+    switch (pl.nch) {
+#define X(n) case n: return launch_stage_mid_t<n>(p, grid, st);
         CFPP_NCH_CASES(X)
 #undef X
     }
@@ -1517,6 +1598,7 @@ int fill_params(const cfpp_neox_dims* d, const cfpp_neox_weights* w, const cfpp_
     p.cache_rows = io->cache_rows;
     p.cos = io->cos; p.sin = io->sin; p.rope_stride = io->rope_stride;
     p.seq_len = io->seq_len; p.d_seq_len = io->d_seq_len;
+    p.seq_cap = (io->d_seq_len && io->max_seq_len > 0) ? io->max_seq_len : io->cache_rows;
     // one (head, split) item per attention wave of the fused launch at most: an item more than that would
     // start only after some wave has finished its first one, and end the attention phase late
     // ... and one attention wave per workgroup is better left without an item when the layer has MLP rows: it then
@@ -1566,11 +1648,17 @@ int run_layer(const Plan& pl, LayerParams& p, int mode, int seq_hint, hipStream_
 
 int run_split(const Plan& pl, LayerParams& p, int seq_hint, hipStream_t st) {
     const int grid = grid_for_streaming(pl);
-    int rc = launch_stage_a(pl, p, grid, st);
+    int rc = launch_stage_qkv(pl, p, grid, st);
     if (rc) return rc;
-    const int bgrid = (p.heads * (split_bound(seq_hint, p.max_split) + 1) + kStreamers - 1) / kStreamers;
-    hipLaunchKernelGGL(k_stage_b, dim3(bgrid), dim3(kStreamers * 64), 0, st, p);
-    if ((rc = launch_check())) return rc;
+    if (p.F > 0) {
+        // attention items beside the MLP-up rows
+        if ((rc = launch_stage_mid(pl, p, grid, st))) return rc;
+    } else {
+        // no MLP in this layer: the attention items alone, one per wave
+        const int bgrid = (p.heads * (split_bound(seq_hint, p.max_split) + 1) + kStreamers - 1) / kStreamers;
+        hipLaunchKernelGGL(k_stage_b, dim3(bgrid), dim3(kStreamers * 64), 0, st, p);
+        if ((rc = launch_check())) return rc;
+    }
     return launch_stage_c(pl, p, grid, st);
 }
 
@@ -1666,6 +1754,7 @@ const char* cfpp_status_str(int s) {
         case CFPP_ERR_ALIGN: return "tensor pointer is not 16-byte aligned";
         case CFPP_ERR_ALIAS: return "an output overlaps an input";
         case CFPP_ERR_STATIC_SCRATCH: return "the layer needs more scratch than the static array of the allocation-free entry point holds";
+        case CFPP_ERR_NOT_INITIALISED: return "cfpp_init() has not run on this device (the allocation-free entry point cannot create the failure-flag word itself)";
         default: break;
     }
     if (s > 0) return hipGetErrorString((hipError_t)s);
@@ -1705,6 +1794,15 @@ int cfpp_neox_layer_decode_static(const cfpp_neox_dims* dims, const cfpp_neox_we
     const WorkspaceLayout L = workspace_layout(*dims);
     if (L.total > kStaticScratchBytes) return CFPP_ERR_STATIC_SCRATCH;
     struct NoAlloc { NoAlloc() { tl_no_alloc = true; } ~NoAlloc() { tl_no_alloc = false; } } guard;
+    {
+        // A failure inside the kernels (an expired wait, a device-side length out of range) is reported through the
+        // pinned status line of the device.  This call may not create it (it allocates nothing), and the status word
+        // inside the scratch array is cleared by the next call: without the line a failure would be lost, so the
+        // call insists on cfpp_init() (or any other launching entry point) having run on this device before.
+        const DeviceInfo& di = device_info();
+        if (!di.ok) return (int)hipErrorNoDevice;
+        if (di.host_status == nullptr) return CFPP_ERR_NOT_INITIALISED;
+    }
     void* ws = nullptr;
     if ((rc = static_scratch_address(&ws))) return rc;
     LayerParams p;
@@ -1801,7 +1899,7 @@ size_t cfpp_llama_plain_workspace_bytes(int32_t hidden, int32_t heads, int32_t h
     const int grid = streaming_grid();
     const int ppm = (hidden + kChunk - 1) / kChunk;
     const size_t units = (size_t)(3 * ppm > grid ? 3 * ppm : grid) + 3 * ppm;     // (panels x slices) never exceeds this
-    return base + align_up(units * kChunk * 4, 256) + align_up((size_t)3 * ppm * 4, 256) + align_up((size_t)hidden * 2, 256);
+    return base + align_up(units * kChunk * 4, 256) + align_up((size_t)3 * ppm * 4, 256);
 }
 int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t workspace_bytes, void* stream) {
     if (!a || !workspace) return CFPP_ERR_NULL;
@@ -1829,10 +1927,7 @@ int cfpp_llama_attention_plain(const cfpp_llama_attn* a, void* workspace, size_t
     const size_t units = (size_t)(3 * ppm > grid ? 3 * ppm : grid) + 3 * ppm;
     float* part = reinterpret_cast<float*>(ws + L.total);
     int* cnt = reinterpret_cast<int*>(ws + L.total + align_up(units * kChunk * 4, 256));
-    half_t* xn = reinterpret_cast<half_t*>(reinterpret_cast<char*>(cnt) + align_up((size_t)3 * ppm * 4, 256));
     auto h = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
-
-    (void)xn;
     CFPP_REFUSE_AFTER_FAILURE();
 
     cfpp_neox_weights w{};
@@ -2016,7 +2111,7 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
 
 int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void* attn_output,
                        const void* mlp_intermediate, const void* w_down, const void* b_down, void* output,
-                       void* workspace, size_t workspace_bytes, void* stream) {
+                       void* /* workspace: not needed */, size_t /* workspace_bytes */, void* stream) {
     int rc = check_dims(dims);
     if (rc) return rc;
     const void* req[] = {input, attn_output, mlp_intermediate, w_down, b_down, output};
@@ -2024,7 +2119,6 @@ int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void
         if (!q) return CFPP_ERR_NULL;
         if (!aligned16(q)) return CFPP_ERR_ALIGN;
     }
-    (void)workspace; (void)workspace_bytes;
     Plan pl;
     if ((rc = make_plan(*dims, &pl))) return rc;
     if (!shape_supported(pl)) return CFPP_ERR_DIMS;
@@ -2060,12 +2154,7 @@ int cfpp_workspace_check(const cfpp_neox_dims* dims, void* workspace, void* stre
 }
 
 int cfpp_device_status(int clear) {
-    DeviceInfo& di = device_info();
-    if (!di.host_status) return 0;
-    volatile int* w = reinterpret_cast<volatile int*>(di.host_status);
-    const int flags = *w;
-    if (clear) *w = 0;
-    return flags;
+    return host_status_flags(device_info(), clear != 0);
 }
 
 int cfpp_one_launch_fits(int grid, int compute_units, int blocks_per_cu) {

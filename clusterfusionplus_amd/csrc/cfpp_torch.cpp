@@ -662,7 +662,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         // 1024*16*16 elements, or None to switch tracing off
         typedef int (*set_trace_fn)(void*);
         set_trace_fn fn = reinterpret_cast<set_trace_fn>(dlsym(RTLD_DEFAULT, "cfpp_debug_set_trace"));
-        TORCH_CHECK(fn != nullptr, "this build of libcfpp.so has no phase tracing (build it with CFPP_TRACE=1)");
+        TORCH_CHECK(fn != nullptr, "the loaded HIP library has no phase tracing: clusterfusionplus_amd/phase_trace.py loads a profiling build before the package");
         if (buf.has_value()) {
             TORCH_CHECK(buf->is_cuda() && buf->scalar_type() == torch::kInt64 && buf->is_contiguous() && buf->numel() >= 1024 * 16 * 16,
                         "trace buffer must be a contiguous int64 GPU tensor with >= 262144 elements");

@@ -80,6 +80,70 @@ def kv_cache_from_hf(key: torch.Tensor, value: torch.Tensor, rows: int, dtype=to
     return kc, vc, S
 
 
+def config_from_hf(hf_config) -> NeoxConfig:
+    """The geometry of a HuggingFace `GPTNeoXConfig` (the fields reference tests/benchmark_decode.py:60-81 reads from the
+    loaded model).  The rotary fraction and base are under `rope_parameters` in current transformers and were
+    `rotary_pct` / `rotary_emb_base` before."""
+    H, nh = int(hf_config.hidden_size), int(hf_config.num_attention_heads)
+    D = H // nh
+    rp = getattr(hf_config, "rope_parameters", None) or {}
+    pct = rp.get("partial_rotary_factor", getattr(hf_config, "rotary_pct", 0.25))
+    base = rp.get("rope_theta", getattr(hf_config, "rotary_emb_base", 10000.0))
+    if not getattr(hf_config, "use_parallel_residual", True):
+        raise ValueError("the decode kernels implement GPT-NeoX's parallel residual only (use_parallel_residual=True)")
+    return NeoxConfig(hidden=H, heads=nh, head_dim=D, rotary_dim=int(D * pct), ffn=int(hf_config.intermediate_size),
+                      n_layers=int(hf_config.num_hidden_layers), vocab=int(hf_config.vocab_size),
+                      eps=float(hf_config.layer_norm_eps), rope_base=float(base))
+
+
+def _hf_layer_kv(past_key_values, l):
+    """Layer l's (key, value) `[1, heads, S, D]` of a transformers cache object or of the legacy tuple of pairs."""
+    if hasattr(past_key_values, "layers"):
+        layer = past_key_values.layers[l]
+        return layer.keys, layer.values
+    if hasattr(past_key_values, "key_cache"):
+        return past_key_values.key_cache[l], past_key_values.value_cache[l]
+    return past_key_values[l][0], past_key_values[l][1]
+
+
+def stack_tensors_from_hf(hf_model, past_key_values, max_rows: int, dtype=torch.float16, device=None):
+    """Everything a whole-model decoder needs, taken from a HuggingFace `GPTNeoXForCausalLM` and the `past_key_values`
+    of its prefill: the hand-off reference tests/benchmark_decode.py:60-119 does by hand (12 tensors per layer,
+    `embed_in`, `final_layer_norm`, `embed_out`, one `[max_rows, H]` K and V cache per layer holding the prefilled
+    positions).  Returns a dict with `cfg`, `layers`, `embed`, `final_ln_w`, `final_ln_b`, `lm_head`, `k_caches`,
+    `v_caches` and `seq_len` (positions already in the caches)."""
+    cfg = config_from_hf(hf_model.config)
+    act = getattr(hf_model.config, "hidden_act", "gelu")
+    if act not in ("gelu_pytorch_tanh", "gelu_new", "gelu_fast", "gelu"):
+        raise ValueError(f"hidden_act {act!r}: the decode kernels compute tanh-GELU")
+    if act == "gelu":
+        import warnings
+        warnings.warn("hidden_act 'gelu' (erf): the decode kernels compute the tanh form, as the reference's kernels do "
+                      "(reference include/5090/pythia_2b8/kernel.cuh:26-49); expect differences of the order of 1e-3")
+    body = hf_model.gpt_neox
+    if len(body.layers) != cfg.n_layers:
+        raise ValueError("config and module disagree on the number of layers")
+
+    def conv(t):
+        t = t.detach().to(dtype)
+        return (t.to(device) if device is not None else t).contiguous()
+    layers = [layer_tensors_from_hf(l, dtype=dtype, device=device) for l in body.layers]
+    k_caches, v_caches, seq = [], [], None
+    for l in range(cfg.n_layers):
+        key, value = _hf_layer_kv(past_key_values, l)
+        kc, vc, n = kv_cache_from_hf(key, value, rows=max_rows, dtype=dtype, device=device)
+        if seq is not None and n != seq:
+            raise ValueError(f"layer {l} holds {n} cached positions, layer 0 holds {seq}")
+        seq = n
+        k_caches.append(kc)
+        v_caches.append(vc)
+    if seq >= max_rows:
+        raise ValueError(f"max_rows ({max_rows}) leaves no cache row for the first generated token ({seq} cached positions)")
+    return {"cfg": cfg, "layers": layers, "embed": conv(body.embed_in.weight),
+            "final_ln_w": conv(body.final_layer_norm.weight), "final_ln_b": conv(body.final_layer_norm.bias),
+            "lm_head": conv(hf_model.get_output_embeddings().weight), "k_caches": k_caches, "v_caches": v_caches, "seq_len": seq}
+
+
 class NeoxDecoder:
     """Greedy batch-1 decoder over device-resident weights and KV caches.
 
@@ -99,6 +163,17 @@ class NeoxDecoder:
         self._stack = native.NeoxStack(cfg.hidden, cfg.heads, cfg.head_dim, cfg.rotary_dim, cfg.ffn, cfg.eps,
                                        packed, embed, final_ln_w, final_ln_b, lm_head, list(k_caches), list(v_caches),
                                        self.cos, self.sin, {"fused": 0, "split": 1}[mode])
+
+    @classmethod
+    def from_hf(cls, hf_model, past_key_values, max_rows: int, device="cuda", mode: str = "fused"):
+        """The prefill -> decode hand-off for a whole model (reference tests/benchmark_decode.py:60-119,147-189): a
+        HuggingFace `GPTNeoXForCausalLM` and the `past_key_values` of its prefill become a decoder whose caches hold the
+        prefilled positions and have room for `max_rows` positions in all.  Returns `(decoder, seq_len)`; continue with
+        `decoder.set_state(first_generated_token, seq_len)` and `graph_steps`."""
+        t = stack_tensors_from_hf(hf_model, past_key_values, max_rows, dtype=torch.float16, device=device)
+        dec = cls(t["cfg"], t["layers"], t["embed"], t["final_ln_w"], t["final_ln_b"], t["lm_head"], t["k_caches"], t["v_caches"],
+                  mode=mode)
+        return dec, t["seq_len"]
 
     def set_state(self, token: int, seq_len: int):
         self._stack.set_state(int(token), int(seq_len))

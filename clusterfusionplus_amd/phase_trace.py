@@ -1,17 +1,36 @@
 """Phase timeline of the fused decoder-layer kernel inside a whole-model decode step.
 
-Needs a profiling build of the HIP library (`python -m clusterfusionplus_amd.build --trace-lib PATH`, then PATH in
-place of libcfpp.so): its fused kernel stores a 100 MHz timestamp per wave at every phase boundary.  This tool runs a
-synthetic model of the given shape, records one eager step, and prints per phase the median over the layers of the
-mean / earliest / latest time (microseconds from the kernel's first wave) over all workgroups.
+Needs a profiling build of the HIP library, kept at a path of its own (it never replaces the product library): its
+fused kernel stores a 100 MHz timestamp per wave at every phase boundary.  This script loads that build before the
+package (both carry the same library name, so the binding resolves to the one already loaded), runs a synthetic model
+of the given shape, records one eager step, and prints per phase the median over the layers of the mean / earliest /
+latest time (microseconds from the kernel's first wave) over all workgroups.  Run it as a script, not with -m (the
+package import would load the product library first):
 
-    python -m clusterfusionplus_amd.phase_trace --model pythia_2b8 --ctx 1024
+    python -m clusterfusionplus_amd.build --trace-lib /tmp/libcfpp_trace.so
+    python clusterfusionplus_amd/phase_trace.py --trace-lib /tmp/libcfpp_trace.so --model pythia_2b8 --ctx 1024
 """
 import argparse
+import ctypes
+import os
 import sys
 
 import numpy as np
 import torch
+
+if __package__ in (None, ""):            # run as a script: make the package importable, but do not import it yet
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+
+def load_trace_library(path):
+    """Loads the profiling build globally, before anything has loaded the product library."""
+    if "clusterfusionplus_amd" in sys.modules:
+        raise RuntimeError("the package is already imported (its product library is loaded): run this file as a script, "
+                           "python clusterfusionplus_amd/phase_trace.py --trace-lib PATH ...")
+    lib = ctypes.CDLL(os.path.abspath(path), mode=ctypes.RTLD_GLOBAL)
+    if not hasattr(lib, "cfpp_debug_set_trace"):
+        raise RuntimeError(f"{path} is not a profiling build (python -m clusterfusionplus_amd.build --trace-lib PATH)")
+    return lib
 
 # slot -> (label, which waves report it)
 SLOTS = [(0, "kernel entry", "all"), (14, "LayerNorm inputs and first weight tile requested", "all"), (15, "own chunk of the input row arrived", "all"),
@@ -24,7 +43,7 @@ SLOTS = [(0, "kernel entry", "all"), (14, "LayerNorm inputs and first weight til
 
 
 def synthetic_decoder(cfg, rows, device):
-    from . import NeoxDecoder
+    from clusterfusionplus_amd import NeoxDecoder
     torch.manual_seed(0)
     H, F = cfg.hidden, cfg.ffn
 
@@ -39,12 +58,14 @@ def synthetic_decoder(cfg, rows, device):
 
 
 def main():
-    from . import PYTHIA_2B8, PYTHIA_6B9, debug_set_trace
     ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--trace-lib", required=True, metavar="PATH", help="the profiling build of the HIP library to load")
     ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8", "llama2_7b_attention"])
     ap.add_argument("--ctx", type=int, default=2048)
     ap.add_argument("--raw", help="also save the raw timestamps of every layer ([layer][workgroup][wave][slot]) as .npy")
     a = ap.parse_args()
+    load_trace_library(a.trace_lib)
+    from clusterfusionplus_amd import PYTHIA_2B8, PYTHIA_6B9, debug_set_trace
     dev = "cuda:0"
     if a.model == "llama2_7b_attention":
         return llama_attention(a, dev)
@@ -84,7 +105,7 @@ def llama_attention(a, dev):
     """The LLaMA-2-7B attention block (fused add + RMSNorm, QKV, attention, O: the fused kernel without an MLP) over eight
     weight sets in turn."""
     import clusterfusion as cf
-    from . import debug_set_trace
+    from clusterfusionplus_amd import debug_set_trace
     H, heads, S = 4096, 32, a.ctx
     torch.manual_seed(0)
 

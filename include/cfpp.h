@@ -48,13 +48,17 @@ typedef enum cfpp_status {
                                   that was checked */
     CFPP_ERR_ALIGN = -8,       /* a tensor pointer is not 16-byte aligned */
     CFPP_ERR_ALIAS = -9,       /* an output overlaps an input it must not overlap */
-    CFPP_ERR_STATIC_SCRATCH = -10  /* cfpp_neox_layer_decode_static: the geometry needs more than cfpp_static_scratch_bytes() */
+    CFPP_ERR_STATIC_SCRATCH = -10, /* cfpp_neox_layer_decode_static: the geometry needs more than cfpp_static_scratch_bytes() */
+    CFPP_ERR_NOT_INITIALISED = -11 /* cfpp_neox_layer_decode_static: cfpp_init() (or another launching entry point) has not
+                                      run on this device yet, so the word that reports device-side failures does not exist */
 } cfpp_status;
 
 /* Layer geometry.  Pythia-2.8B = {2560,32,80,20,10240,1e-5}, Pythia-6.9B = {4096,32,128,32,16384,1e-5}
  * (reference include/5090/pythia_2b8/config.h:6-12, include/5090/pythia_6b9/config.h:6-12).
- * Supported: hidden == heads*head_dim, hidden % 8 == 0, hidden <= 8192, head_dim % 8 == 0,
- * head_dim <= 128, rotary_dim even and <= head_dim, ffn % 8 == 0. */
+ * Supported: hidden == heads*head_dim, hidden % 8 == 0, hidden <= 4096, head_dim % 8 == 0,
+ * head_dim <= 128, rotary_dim even and <= head_dim, ffn % 8 == 0, and (ceil(hidden / 512), ceil(ceil(ffn / 512) / 4))
+ * one of (1,1) (2,2) (4,4) (5,5) (8,8) (8,6): the shapes the kernels are instantiated for (hidden 512, 1024, 2048,
+ * 2560, 4096 with ffn = 4 hidden; hidden 4096 with ffn 11008); anything else returns CFPP_ERR_DIMS. */
 typedef struct cfpp_neox_dims {
     int32_t hidden, heads, head_dim, rotary_dim, ffn;
     float eps;
@@ -87,7 +91,8 @@ typedef struct cfpp_neox_io {
     int32_t rope_stride;
     int32_t seq_len;
     const int32_t* d_seq_len;
-    int32_t max_seq_len;     /* upper bound used to size the KV split when d_seq_len is given; 0 = cache_rows */
+    int32_t max_seq_len;     /* with d_seq_len: the largest length the launches are sized for (0 = cache_rows); a device-side
+                                length beyond it raises the failure flag instead of being attended */
     void* attn_output;       /* split API only: [H] fp16 = W_o attn + b_o */
     void* mlp_intermediate;  /* split API only: [F] fp16 = gelu(W_up ln2(x) + b_up) */
 } cfpp_neox_io;
@@ -119,9 +124,11 @@ int cfpp_neox_layer_decode(const cfpp_neox_dims* dims, const cfpp_neox_weights* 
  * Pythia models fit).  All calls on one device share the one array: calls on the same stream are ordered and fine,
  * calls that overlap in time on one device (two streams, two threads) race and give wrong results.  Every call
  * first clears the array's counters and flags with a small kernel (it keeps the previous call's contents), then
- * runs the same kernels as cfpp_neox_layer_decode: identical results, bit for bit.  The first call on a device looks
- * up the device's copy of the array; call cfpp_init() beforehand (device current) when that first call may sit
- * inside a graph capture. */
+ * runs the same kernels as cfpp_neox_layer_decode: identical results, bit for bit.  cfpp_init() (device current) must
+ * have run on the device before the first call: it creates the pinned word through which a device-side failure of
+ * these launches is reported (cfpp_device_status; the status word inside the array is cleared by the next call and
+ * cannot serve), which this entry point may not allocate itself.  Without it the call launches nothing and returns
+ * CFPP_ERR_NOT_INITIALISED.  (Any other launching entry point of the library creates the word as well.) */
 int cfpp_neox_layer_decode_static(const cfpp_neox_dims* dims, const cfpp_neox_weights* w, const cfpp_neox_io* io,
                                   int mode, void* stream);
 size_t cfpp_static_scratch_bytes(void);
@@ -236,7 +243,8 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
 
 /* Second half: output = input + attn_output + W_down mlp_intermediate + b_down.
  * Replaces pythia_2b8_mlp_only_sm120 (reference include/pybind.cpp:174-180;
- * pythia_kernel_dispatch_split.cu:364-426). */
+ * pythia_kernel_dispatch_split.cu:364-426).  `workspace` / `workspace_bytes` are not used (the call needs no scratch
+ * memory; NULL / 0 are fine): they keep the argument list of the two halves alike. */
 int cfpp_neox_mlp_down(const cfpp_neox_dims* dims, const void* input, const void* attn_output,
                        const void* mlp_intermediate, const void* w_down, const void* b_down, void* output,
                        void* workspace, size_t workspace_bytes, void* stream);
@@ -276,7 +284,7 @@ int cfpp_workspace_check(const cfpp_neox_dims* dims, void* workspace, void* stre
 int cfpp_ctx_check(int family, int64_t id, void* stream);
 
 /* Failure flags raised by any launch on the current device since they were last cleared (bit 0: a bounded
- * device-side wait expired; bit 1: a device-side seq_len was out of range), read from a word of pinned host memory
+ * device-side wait expired; bit 1: a device-side seq_len was out of range), read from pinned host memory (one word per flag)
  * that the kernels write on failure: no device synchronisation, callable at any time; flags of launches still
  * running are seen once they got there.  `clear` != 0 resets the word.  While it is non-zero every launching entry
  * point returns CFPP_ERR_DEVICE.  No counterpart in the reference (which checks no error at all). */

@@ -41,8 +41,9 @@ def test_status_strings_and_version(lib):
     lib.cfpp_status_str.restype = ctypes.c_char_p
     lib.cfpp_version.restype = ctypes.c_char_p
     assert lib.cfpp_status_str(0) == b"ok"
-    seen = {lib.cfpp_status_str(-i) for i in range(1, 11)}
-    assert len(seen) == 10 and b"unknown status" not in seen
+    seen = {lib.cfpp_status_str(-i) for i in range(1, 12)}
+    assert len(seen) == 11 and b"unknown status" not in seen
+    assert lib.cfpp_status_str(-12) == b"unknown status"
     assert b"gfx950" in lib.cfpp_version()
 
 
@@ -142,6 +143,27 @@ def test_static_entry_point_argument_errors_launch_nothing(lib):
     assert lib.cfpp_neox_layer_decode_static(ctypes.byref(wide), None, None, 0, None) == -10
     lib.cfpp_status_str.restype = ctypes.c_char_p
     assert b"static" in lib.cfpp_status_str(-10)
+    assert b"cfpp_init" in lib.cfpp_status_str(-11)
+    # a valid geometry gets as far as the device set-up and no further: without a GPU that is a HIP error (> 0), with
+    # one it is -11 until cfpp_init() has created the failure-flag word (NULL tensors are looked at after that)
+    import torch
+    rc = lib.cfpp_neox_layer_decode_static(ctypes.byref(d), None, None, 0, None)
+    assert (rc > 0) if not torch.cuda.is_available() else rc in (-11, -1)
+
+
+def test_shapes_without_an_instantiation_are_refused(lib):
+    """Only the (hidden chunks, MLP-down chunks) pairs the kernels are instantiated for are accepted; the workspace size
+    is defined for any valid geometry, the launching calls refuse the others before touching the device."""
+    ws = ctypes.c_void_p(1 << 20)
+    w = (ctypes.c_void_p * 12)(*([4096] * 12))
+    for hidden, heads, hd, ffn in ((1536, 12, 128, 6144), (3072, 24, 128, 12288), (3584, 28, 128, 14336), (4096, 32, 128, 8192)):
+        d = Dims(hidden, heads, hd, 32, ffn, 1e-5)
+        io = NeoxIo(input=4096, output=4096, k_new=4096, v_new=4096, k_cache=4096, v_cache=4096, cache_rows=10, cos=4096, sin=4096,
+                    rope_stride=0, seq_len=0, d_seq_len=None, max_seq_len=0, attn_output=None, mlp_intermediate=None)
+        assert lib.cfpp_neox_layer_decode(ctypes.byref(d), w, ctypes.byref(io), 0, ws, ctypes.c_size_t(8 << 20), None) == -2, hidden
+    buf = ctypes.create_string_buffer(64)
+    ptr = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.cfpp_neox_lm_head(1536, 100, ctypes.c_float(1e-5), ptr, ptr, ptr, ptr, ctypes.cast(buf, ctypes.POINTER(ctypes.c_float)), None) == -2
 
 
 class LlamaBatch(ctypes.Structure):
