@@ -26,6 +26,9 @@ HIPCC_FLAGS = [
     # packed-fp32 arithmetic stays off in device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # no contraction of a*b + c by the compiler: every fused multiply-add of the kernels is written out, so that a device
+    # function rounds the same way in every kernel it is inlined into (split == fused, bit for bit)
+    "-ffp-contract=off",
     # one name for the product build and for profiling builds kept elsewhere: a process that has loaded either one
     # resolves the binding's dependency on "libcfpp.so" to it
     "-Wl,-soname,libcfpp.so",

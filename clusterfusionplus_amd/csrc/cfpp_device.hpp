@@ -84,6 +84,7 @@ struct LayerParams {
     const int* tag_src;     // launch tags from a counter the caller advances between launches (null: from kBarGen)
     int tag_mul, tag_add;   // tag = tag_src[0] * tag_mul + tag_add + 1
     int arrival_agents;     // an idle attention wave carries the streaming waves' MLP-up arrivals to the device-wide counters
+    int up_wgs;             // split mode: workgroups that share the MLP-up rows of the middle launch (it may have more, for attention items)
     // layer family switches (defaults = GPT-NeoX): RMSNorm instead of LayerNorm; where head h's raw q, k, v sit in
     // qkv_raw (NeoX interleaves [h][q|k|v][D]: stride 3D, offsets D and 2D; LLaMA stacks [q;k;v]: stride D,
     // offsets H and 2H); whether split 0 appends the new K/V row to the caches
@@ -132,6 +133,23 @@ __device__ __forceinline__ void trace_mark(const LayerParams&, int) {}
 // ------------------------------------------------------------------------------------------------
 // loads / conversions
 // ------------------------------------------------------------------------------------------------
+// The parameter block of a kernel (several hundred bytes) does not fit the scalar registers, so the compiler loads it
+// piecemeal, where each piece is first needed, and waits for each piece: at the start of a launch every one of those
+// loads misses the (just invalidated) scalar cache, and half a dozen dependent misses in a row stood in front of the
+// first weight request.  Reading one word of every 64-byte line of the kernel-argument segment up front, all in
+// flight together, turns them into one miss; everything after that hits.
+template <int BYTES>
+__device__ __forceinline__ void touch_kernel_arguments() {
+    typedef __attribute__((address_space(4))) const int ConstInt;
+    ConstInt* ka = (ConstInt*)__builtin_amdgcn_kernarg_segment_ptr();
+    int acc = 0;
+#pragma unroll
+    for (int off = 0; off < BYTES; off += 64) acc ^= ka[off / 4];
+    asm volatile("; kernel arguments resident (%0)" ::"s"(acc));
+}
+// bytes of the kernel-argument segment of a kernel whose only explicit argument is a LayerParams (+ the hidden ones
+// the runtime appends: grid and block sizes)
+constexpr int kLayerKernargBytes = 448;
 __device__ __forceinline__ u32x4 ld_stream16(const void* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }
@@ -223,10 +241,16 @@ __device__ __forceinline__ int first_lane(int v) { return __builtin_amdgcn_readf
 // ------------------------------------------------------------------------------------------------
 // math
 // ------------------------------------------------------------------------------------------------
+// The library is compiled with -ffp-contract=off and every fused multiply-add is written out (fmadd below): the
+// per-stage kernels and the one-launch kernel inline the same functions into different surroundings, and a compiler
+// that is free to contract a*b + c*d either way (or not at all) can round the same expression differently in two
+// kernels - enough to flip an fp16 rounding of a rotated K value once in a few thousand, which the bit-exact
+// split == fused checks at full model depth catch.
+__device__ __forceinline__ float fmadd(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 // tanh-GELU, 0.5 x (1 + tanh(sqrt(2/pi)(x + 0.044715 x^3))) with tanh(u) = 1 - 2/(1 + e^{2u}) on the
 // native exp2 (reference include/5090/pythia_2b8/kernel.cuh:26-49 builds the same from ex2.approx).
 __device__ __forceinline__ float gelu_tanh(float x) {
-    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    const float u = 0.7978845608028654f * fmadd(0.044715f * x * x, x, x);
     const float e = __builtin_amdgcn_exp2f(u * 2.8853900817779268f);   // e^{2u}
     const float t = 1.0f - 2.0f / (1.0f + e);
     return 0.5f * x * (1.0f + t);
@@ -446,7 +470,7 @@ __device__ __forceinline__ void ln_coop_finish(const LnOwn<NCH, NW>& o, const No
             unpack8(o.rx[k], xv);
             if (i * kChunk + lane * 8 < H) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) { const float d = xv[j] - mean; q += d * d; }
+                for (int j = 0; j < 8; ++j) { const float d = xv[j] - mean; q = fmadd(d, d, q); }
             }
             q = wave_sum(q);
             if (lane == 0) sh.part[1][i] = q;
@@ -465,16 +489,24 @@ __device__ __forceinline__ void ln_coop_finish(const LnOwn<NCH, NW>& o, const No
             float xv[8], g[8], b[8], y[8];
             unpack8(o.rx[k], xv); unpack8(o.rw1[k], g); unpack8(o.rb1[k], b);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) y[j] = in ? (xv[j] - mean) * rstd * g[j] + b[j] : 0.f;
+            for (int j = 0; j < 8; ++j) y[j] = in ? fmadd((xv[j] - mean) * rstd, g[j], b[j]) : 0.f;
             *reinterpret_cast<u32x4*>(&sh.y[0][i * kChunk + lane * 8]) = pack8(y);
             if (TWO) {
                 unpack8(o.rw2[k], g); unpack8(o.rb2[k], b);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) y[j] = in ? (xv[j] - mean) * rstd * g[j] + b[j] : 0.f;
+                for (int j = 0; j < 8; ++j) y[j] = in ? fmadd((xv[j] - mean) * rstd, g[j], b[j]) : 0.f;
                 *reinterpret_cast<u32x4*>(&sh.y[1][i * kChunk + lane * 8]) = pack8(y);
             }
         }
     }
+    __syncthreads();
+}
+
+// For waves of the workgroup that take no part in the norm (they hold other work in flight): the workgroup barriers
+// of ln_coop_finish, nothing else.
+__device__ __forceinline__ void ln_coop_bystander(const NormSpec& ns) {
+    if (!ns.rms) __syncthreads();
+    __syncthreads();
     __syncthreads();
 }
 
@@ -887,7 +919,7 @@ __device__ __forceinline__ void rope_finish(const RopeRaw& r, int d0, int rot, c
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const float pr = PAIRS ? r.a[j ^ 1] : r.pr[j];          // GPT-J: the neighbour is one of the lane's own eight dims
-        out[j] = act ? (d0 + j < rot ? r.a[j] * rc.c[j] + pr * rc.sg[j] : r.a[j]) : 0.f;
+        out[j] = act ? (d0 + j < rot ? fmadd(r.a[j], rc.c[j], pr * rc.sg[j]) : r.a[j]) : 0.f;
     }
 }
 __device__ __forceinline__ void raw_load8(const float* __restrict__ v, int d0, bool act, float (&out)[8]) {
@@ -1003,7 +1035,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
         if (grp == 0) {
             float s = 0.f;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) s += q[j] * p.qscale * kf[j];
+            for (int j = 0; j < 8; ++j) s = fmadd(q[j] * p.qscale, kf[j], s);
             s = row16_sum(s);
             m = s; l = 1.f;
 #pragma unroll
@@ -1034,7 +1066,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
                 unpack8(kv.k[t], kf);
                 float d = 0.f;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) d += q[j] * kf[j];
+                for (int j = 0; j < 8; ++j) d = fmadd(q[j], kf[j], d);
                 d = row16_sum(d);
                 s[t] = (r + t * 4 < end) ? d : kNegBig;
                 mt = fmaxf(mt, s[t]);
@@ -1050,7 +1082,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
                 unpack8(kv.v[t], vf);
                 l += pt;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) acc[j] += pt * vf[j];
+                for (int j = 0; j < 8; ++j) acc[j] = fmadd(pt, vf[j], acc[j]);
             }
             m = mt;
         };
@@ -1148,8 +1180,8 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
                 const int i = in ? i0 + u : 0;
                 const float sc = in ? rl(sci, i) : 0.f;
                 L += in ? rl(lsi, i) : 0.f;
-                A0 += a0[u] * sc;
-                A1 += a1[u] * sc;
+                A0 = fmadd(a0[u], sc, A0);
+                A1 = fmadd(a1[u], sc, A1);
             }
         }
         if (dact) {

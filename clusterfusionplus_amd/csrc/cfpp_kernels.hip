@@ -136,6 +136,7 @@ __device__ __forceinline__ void up_team_rows(const LayerParams& p, const half2_t
 //   k_stage_c     O projection on four waves beside the MLP-down rows on the other four, residual.
 template <int NCH, int NW, bool EX>
 __global__ __launch_bounds__(NW * 64) void k_stage_qkv(LayerParams p) {
+    touch_kernel_arguments<kLayerKernargBytes>();
     __shared__ float park_mem[NW][kParkRows];
     __shared__ LnShared<NCH> lns;
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
@@ -153,45 +154,46 @@ __global__ __launch_bounds__(NW * 64) void k_stage_qkv(LayerParams p) {
     qkv_rows<NCH, EX>(p, xr, qw, lane, t0, park);
 }
 
-// MLP-up rows on the streaming waves, attention items on the other four; wave hw of workgroup b takes the items
-// b + hw G, + 4 G, ... (any number of items: nothing here waits for another workgroup).
+// MLP-up rows on the streaming waves of the first p.up_wgs workgroups (one per compute unit), attention items on the
+// other four waves: wave hw of workgroup b takes item b + hw G.  The host sizes the grid so that every item has a wave
+// (workgroups beyond p.up_wgs have no rows and only run items; nothing here waits for another workgroup, so they may
+// start whenever a compute unit has room).  The two halves share nothing but the workgroup barriers of the norm, which
+// the attention waves only pass through with their item's loads in flight.  (One item per wave and no loop: a loop
+// around the item makes the compiler keep more than 256 registers alive.)
 template <int NCH, bool EX>
 __global__ __launch_bounds__(2 * kStreamers * 64) void k_stage_mid(LayerParams p) {
+    touch_kernel_arguments<kLayerKernargBytes>();
     __shared__ float park_mem[kStreamers][kParkRows];
     __shared__ LnShared<NCH> lns;
-    constexpr int NW = 2 * kStreamers;
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
     const int G = gridDim.x, b = blockIdx.x;
-    const int hw = wave - kStreamers;
-    const SeqLen sl = load_seq_len(p);
-    const int nsplit = effective_split(p, sl.S), per_head = items_per_head(nsplit);
-    const int nitems = p.heads * per_head;
-    AttnItem it;
-    int item = b + hw * G;
-    // an attention wave's first item is requested before the LayerNorm (it needs none of it) ...
-    if (hw >= 0 && item < nitems) attn_prefetch(p, it, item / per_head, item % per_head, nsplit, sl, lane);
-    // ... the post-attention LayerNorm of the input row, by all eight waves (slot 0 holds it: only one row is needed here)
+    const SeqLen sl = load_seq_len(p);      // by every wave: thread 0 of workgroup 0 reports a length that is out of range
+    // the post-attention LayerNorm of the input row (slot 0 holds it: only one row is needed here)
     NormSpec ns = norm_spec(p);
     ns.w1 = p.ln2_w; ns.b1 = p.ln2_b;
-    LnOwn<NCH, NW> own;
-    ln_coop_load<NCH, NW, false>(own, ns, wave, lane);
-    __builtin_amdgcn_sched_barrier(0);
-    RowTile<NCH, kUpRpi> u0;
-    const RowWalk uw = row_walk<kUpRpi>(b * kStreamers + (hw < 0 ? wave : 0), G * kStreamers, 0, hw < 0 ? p.F : 0);
-    if (hw < 0) up_prefetch<NCH, EX>(p, uw, lane, u0);
-    ln_coop_finish<NCH, NW, false>(own, ns, lns, wave, lane);
-    if (hw < 0) {
+    if (wave < kStreamers) {
+        LnOwn<NCH, kStreamers> own;
+        ln_coop_load<NCH, kStreamers, false>(own, ns, wave, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        RowTile<NCH, kUpRpi> u0;
+        const bool rows = b < p.up_wgs;
+        const RowWalk uw = row_walk<kUpRpi>((rows ? b : 0) * kStreamers + wave, p.up_wgs * kStreamers, 0, rows ? p.F : 0);
+        up_prefetch<NCH, EX>(p, uw, lane, u0);
+        ln_coop_finish<NCH, kStreamers, false>(own, ns, lns, wave, lane);
         RowPark park{park_mem[wave], 0};
         half2_t xr[NCH][4];
         ln_fetch<NCH>(lns, 0, lane, xr);
         up_rows<NCH, EX>(p, xr, uw, lane, u0, park);
     } else {
+        const int hw = wave - kStreamers;
+        const int nsplit = effective_split(p, sl.S), per_head = items_per_head(nsplit);
+        const int nitems = p.heads * per_head;
+        AttnItem it;
+        int item = b + hw * G;
+        if (item < nitems) attn_prefetch(p, it, item / per_head, item % per_head, nsplit, sl, lane);
+        ln_coop_bystander(ns);
         __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
-        while (item < nitems) {
-            attention_item(p, it, lane, 0, 0);
-            item += kStreamers * G;
-            if (item < nitems) attn_prefetch(p, it, item / per_head, item % per_head, nsplit, sl, lane);
-        }
+        if (item < nitems) attention_item(p, it, lane, 0, 0);
     }
 }
 
@@ -199,6 +201,7 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_stage_mid(LayerParams p
 // A tile is the pair (gate row r, up row r + F); a wave owns a contiguous range of pairs.
 template <int NCH, bool EX>
 __global__ __launch_bounds__(kStreamers * 64) void k_gated_up(LayerParams p) {
+    touch_kernel_arguments<kLayerKernargBytes>();
     __shared__ float park_mem[kStreamers][kParkRows];
     __shared__ LnShared<NCH> lns;
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
@@ -230,6 +233,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_up(LayerParams p) {
 // workgroup per compute unit, all co-resident; launch tag from the generation word, published again at the end.
 template <int NCH, int CPD, bool EX>
 __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
+    touch_kernel_arguments<kLayerKernargBytes>();
     __shared__ float park_mem[kStreamers][kParkRows];
     __shared__ LnShared<NCH> lns;
     __shared__ StageCShared shc;
@@ -283,6 +287,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
 
 // one (head, split) item per wave
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_b(LayerParams p) {
+    touch_kernel_arguments<kLayerKernargBytes>();
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
     const SeqLen sl = load_seq_len(p);
     const int nsplit = effective_split(p, sl.S), per_head = items_per_head(nsplit);
@@ -296,6 +301,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_b(LayerParams p) {
 
 template <int NCH, int CPD>
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
+    touch_kernel_arguments<kLayerKernargBytes>();
     __shared__ StageCShared sh;
     const int wave = first_lane(threadIdx.x >> 6);
     const StageC c = make_stage_c(p);
@@ -305,6 +311,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_stage_c(LayerParams p) {
 // other four (all eight when there is no MLP-down pass).  Which wave computes a row does not change its value.
 template <int NCH, int CPD>
 __global__ __launch_bounds__(2 * kStreamers * 64) void k_stage_c8(LayerParams p) {
+    touch_kernel_arguments<kLayerKernargBytes>();
     __shared__ StageCShared sh;
     const int wave = first_lane(threadIdx.x >> 6);
     const StageC c = make_stage_c(p);
@@ -540,11 +547,14 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
 // one layer, parameters in the kernel arguments
 template <int NCH, int CPD, bool EX, bool BYX>
 __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
+    touch_kernel_arguments<kLayerKernargBytes>();
     __shared__ FusedLds<NCH> lds;
     // the flag value of this launch is gen + 1: requested first, needed at the first event.  It comes from the
     // generation the previous launch on this workspace published, or from a counter that the caller advances
     // between launches (a whole-model step: step counter x layers + layer), which saves the publishing.
-    const int gen = p.tag_src != nullptr ? p.tag_src[0] * p.tag_mul + p.tag_add : counter_peek(p.bar + kBarGen);
+    // (a vector load, not waited for until the first event needs the tag)
+    const int gen = counter_peek(p.tag_src != nullptr ? p.tag_src : p.bar + kBarGen) * (p.tag_src != nullptr ? p.tag_mul : 1) +
+                    (p.tag_src != nullptr ? p.tag_add : 0);
     fused_layer<NCH, CPD, EX, BYX>(p, gen, lds);
 }
 
@@ -564,6 +574,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __res
                                                       const half_t* __restrict__ ln_w, const half_t* __restrict__ ln_b,
                                                       const half_t* __restrict__ W, int vocab, float* __restrict__ logits,
                                                       float* __restrict__ best_val, int* __restrict__ best_idx) {
+    touch_kernel_arguments<128>();
     constexpr int NWV = kStreamers;
     __shared__ float sv[NWV];
     __shared__ int si[NWV];
@@ -715,7 +726,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_gemv(BatchGemv a) {
                     if (in && a.sum_out != nullptr && blockIdx.x == 0) *reinterpret_cast<u32x4*>(a.sum_out + base + col) = r;
                 }
 #pragma unroll
-                for (int j = 0; j < 8; ++j) ss += v[i][j] * v[i][j];
+                for (int j = 0; j < 8; ++j) ss = fmadd(v[i][j], v[i][j], ss);
             }
             float rstd = 1.f;
             if (a.norm_w != nullptr) rstd = 1.0f / sqrtf(wave_sum(ss) / (float)a.K + a.eps);
@@ -1028,7 +1039,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_batch_norm(BatchNorm a) {
             if (in) *reinterpret_cast<u32x4*>(a.sum_out + base + col) = r;
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ss += v[i][j] * v[i][j];
+        for (int j = 0; j < 8; ++j) ss = fmadd(v[i][j], v[i][j], ss);
     }
     const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)a.K + a.eps);
 #pragma unroll
@@ -1085,7 +1096,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gemv_t(GemvT a) {
             float f[8];
             unpack8(ld16(a.x + c0), f);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) ss += f[j] * f[j];
+            for (int j = 0; j < 8; ++j) ss = fmadd(f[j], f[j], ss);
         }
         rstd = 1.0f / sqrtf(wave_sum(ss) / (float)a.K + a.eps);
     }
@@ -1107,7 +1118,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gemv_t(GemvT a) {
                 float f[8];
                 unpack8(w[u], f);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) acc[j] += xk * f[j];
+                for (int j = 0; j < 8; ++j) acc[j] = fmadd(xk, f[j], acc[j]);
             }
         }
     }
@@ -1152,6 +1163,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gemv_t(GemvT a) {
 
 // stage B with GPT-J pairing of the rotary dims
 __global__ __launch_bounds__(kStreamers * 64) void k_stage_b_pairs(LayerParams p) {
+    touch_kernel_arguments<kLayerKernargBytes>();
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
     const SeqLen sl = load_seq_len(p);
     const int nsplit = effective_split(p, sl.S), per_head = items_per_head(nsplit);
@@ -1446,12 +1458,17 @@ int launch_fused_t(const LayerParams& p, int grid, hipStream_t st) {
 template <int NCH, int CPD>
 bool fused_fits_t(const LayerParams& p, int grid) { return one_launch_fits(fused_fn<NCH, CPD>(p, grid), 2 * kStreamers * 64, grid); }
 
-// hidden chunks that occur in CFPP_SHAPE_CASES below
+// hidden chunks that occur in CFPP_SHAPE_CASES below (both lists can be narrowed on the compiler's command line for a
+// quick experimental build; the shapes left out are then refused with CFPP_ERR_DIMS)
+#ifndef CFPP_NCH_CASES
 #define CFPP_NCH_CASES(X) X(1) X(2) X(4) X(5) X(8)
+#endif
 // (hidden chunks, MLP-down chunks per streaming wave).  The Pythia family has ffn = 4 hidden, so both
 // numbers coincide: 512 -> (1,1), 768/1024 -> (2,2), 2048 -> (4,4), 2560 -> (5,5), 4096 -> (8,8);
 // (8,6) is hidden 4096 with ffn 11008
+#ifndef CFPP_SHAPE_CASES
 #define CFPP_SHAPE_CASES(X) X(1, 1) X(2, 2) X(4, 4) X(5, 5) X(8, 8) X(8, 6)
+#endif
 
 int launch_stage_qkv(const Plan& pl, const LayerParams& p, int grid, hipStream_t st) {
     switch (pl.nch) {
@@ -1650,12 +1667,15 @@ int run_split(const Plan& pl, LayerParams& p, int seq_hint, hipStream_t st) {
     const int grid = grid_for_streaming(pl);
     int rc = launch_stage_qkv(pl, p, grid, st);
     if (rc) return rc;
+    // one attention wave per (head, split) item
+    const int bgrid = (p.heads * (split_bound(seq_hint, p.max_split) + 1) + kStreamers - 1) / kStreamers;
     if (p.F > 0) {
-        // attention items beside the MLP-up rows
-        if ((rc = launch_stage_mid(pl, p, grid, st))) return rc;
+        // attention items beside the MLP-up rows: the rows on one workgroup per compute unit, more workgroups (items
+        // only) when there are more items than that gives attention waves
+        p.up_wgs = grid;
+        if ((rc = launch_stage_mid(pl, p, bgrid > grid ? bgrid : grid, st))) return rc;
     } else {
-        // no MLP in this layer: the attention items alone, one per wave
-        const int bgrid = (p.heads * (split_bound(seq_hint, p.max_split) + 1) + kStreamers - 1) / kStreamers;
+        // no MLP in this layer: the attention items alone
         hipLaunchKernelGGL(k_stage_b, dim3(bgrid), dim3(kStreamers * 64), 0, st, p);
         if ((rc = launch_check())) return rc;
     }
