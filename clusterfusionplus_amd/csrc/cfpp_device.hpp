@@ -356,8 +356,16 @@ __device__ __forceinline__ StatusSink status_sink(const LayerParams& p) { return
 // attention items in split mode).  Anything else raises kStatusSeq; the step then runs on a clamped length without
 // appending, so that no access leaves the caches or the tables, and its results mean nothing.
 struct SeqLen { int S; bool ok; };
-__device__ __forceinline__ SeqLen load_seq_len(const LayerParams& p) {
-    int S = p.d_seq_len ? *p.d_seq_len : p.seq_len;
+// The length in device memory is requested first thing in a kernel (seq_len_request; the word of the workspace that is
+// read instead when there is none keeps the load unconditional: a conditional load is waited for where the branches join)
+// and looked at where it is needed (seq_len_check).  Requested where it is needed, after the norm, it made every wave wait
+// for one more memory round trip with its first weight tile already used up and nothing else in flight.
+__device__ __forceinline__ int seq_len_request(const LayerParams& p) {
+    const int* src = p.d_seq_len ? p.d_seq_len : p.bar;
+    return *src;
+}
+__device__ __forceinline__ SeqLen seq_len_check(const LayerParams& p, int requested) {
+    int S = p.d_seq_len ? requested : p.seq_len;
     int limit = (p.d_seq_len != nullptr || p.rope_stride > 0) ? p.cache_rows - 1 : p.cache_rows;
     if (p.d_seq_len != nullptr && p.seq_cap < limit) limit = p.seq_cap;
     const bool ok = S >= 0 && S <= limit;
@@ -367,6 +375,7 @@ __device__ __forceinline__ SeqLen load_seq_len(const LayerParams& p) {
     }
     return SeqLen{S, ok};
 }
+__device__ __forceinline__ SeqLen load_seq_len(const LayerParams& p) { return seq_len_check(p, seq_len_request(p)); }
 // KV splits per head for a sequence length: about kSplitRows cache rows per item
 __device__ __forceinline__ int effective_split(const LayerParams& p, int S) {
     int n = (S + kSplitRows - 1) / kSplitRows;
@@ -396,7 +405,7 @@ struct LnShared {
 template <int NCH, int NW>
 struct LnOwn {
     static constexpr int OWN = (NCH + NW - 1) / NW;
-    u32x4 rx[OWN], rw1[OWN], rb1[OWN], rw2[OWN], rb2[OWN];
+    u32x4 rx[OWN], ra[OWN], rw1[OWN], rb1[OWN], rw2[OWN], rb2[OWN];      // ra: the second input row (x_add), if there is one
 };
 
 // What the cooperative norm needs to know about its inputs.
@@ -424,24 +433,31 @@ __device__ __forceinline__ void ln_coop_load(LnOwn<NCH, NW>& o, const NormSpec& 
             o.rw2[k] = (in && ns.w2) ? ld16(ns.w2 + col) : z;
             o.rb2[k] = (in && ns.b2) ? ld16(ns.b2 + col) : z;
         }
-        if (ns.x_add != nullptr) {
-            // x <- fp16(x + x_add), as the reference's fused add + RMSNorm does (reference
-            // include/5090/llama/kernel_sglang.cuh:98-105).  The sum is stored by stage C, once every
-            // workgroup has read both rows: x_sum_out may be x_add itself.
-            const u32x4 ra = in ? ld16(ns.x_add + col) : z;
-            float a[8], b[8];
-            unpack8(o.rx[k], a); unpack8(ra, b);
+        // the second input row, if there is one, is only requested here (without one, the first is requested again and
+        // dropped): adding it up right away would make the wave wait for both rows before anything else can be requested
+        o.ra[k] = in ? ld16((ns.x_add != nullptr ? ns.x_add : ns.x) + col) : z;
+    }
+}
+// x <- fp16(x + x_add), as the reference's fused add + RMSNorm does (reference include/5090/llama/kernel_sglang.cuh:98-105).
+// The sum is stored by stage C, once every workgroup has read both rows: x_sum_out may be x_add itself.
+template <int NCH, int NW>
+__device__ __forceinline__ void ln_coop_add(LnOwn<NCH, NW>& o, const NormSpec& ns) {
+    if (ns.x_add == nullptr) return;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) a[j] += b[j];
-            o.rx[k] = pack8(a);
-        }
+    for (int k = 0; k < LnOwn<NCH, NW>::OWN; ++k) {
+        float a[8], b[8];
+        unpack8(o.rx[k], a); unpack8(o.ra[k], b);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a[j] += b[j];
+        o.rx[k] = pack8(a);
     }
 }
 
 // Every wave of the workgroup must call this (workgroup barriers inside).
 template <int NCH, int NW, bool TWO>
-__device__ __forceinline__ void ln_coop_finish(const LnOwn<NCH, NW>& o, const NormSpec& ns, LnShared<NCH>& sh, int wave, int lane) {
+__device__ __forceinline__ void ln_coop_finish(LnOwn<NCH, NW>& o, const NormSpec& ns, LnShared<NCH>& sh, int wave, int lane) {
     constexpr int OWN = LnOwn<NCH, NW>::OWN;
+    ln_coop_add<NCH, NW>(o, ns);
     const int H = ns.H;
     float mean = 0.f;
     if (!ns.rms) {
@@ -552,6 +568,17 @@ __device__ __forceinline__ void load_row_tile(RowTile<NCH, RPI>& t, const half_t
             }
         }
     }
+}
+
+// The first tile of a wave's row range, requested ahead of something slow (a norm, an event) WITHOUT a branch around the
+// loads: a wave that has no tile requests row 0 (and drops it).  With `if (ntiles > 0)` around them, the compiler's
+// wait-count bookkeeping takes the shorter path at the join behind the branch: the next wait for anything older
+// (the norm's inputs) then waits for the whole tile as well.
+template <int NCH, int RPI, bool EXACT>
+__device__ __forceinline__ void prefetch_row_tile(RowTile<NCH, RPI>& t, const half_t* __restrict__ W, int K, int first, int stride,
+                                                  int end, int ntiles, int lane) {
+    const bool any = ntiles > 0;
+    load_row_tile<NCH, RPI, EXACT>(t, W, K, any ? first : 0, stride, any ? end : 1, lane);
 }
 
 // chunk i of the weight row at rp (same addressing as load_row_tile)
@@ -1360,18 +1387,25 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
     for (int b0 = r0; b0 < r1; b0 += kRowBatch) {
         const int b1 = (b0 + kRowBatch < r1) ? b0 + kRowBatch : r1;
         // what the epilogue of this batch adds to the dot products are inputs of the layer: requested now, so that the
-        // threads that finish the rows do not start a memory round trip after the last barrier
-        float e_b1 = 0.f, e_b2 = 0.f, e_x0 = 0.f, e_x1 = 0.f, e_sa = 0.f, e_sb = 0.f;
-        if ((int)threadIdx.x < b1 - b0) {
-            const int r = b0 + (int)threadIdx.x;
-            if (c.bias1) e_b1 = (float)c.bias1[r];
-            if (c.bias2) e_b2 = (float)c.bias2[r];
-            if (c.base0) e_x0 = (float)c.base0[r];
-            if (c.base1) e_x1 = (float)c.base1[r];
-            if (c.sum_b != nullptr || c.add_sum) {
-                e_sa = (float)c.sum_a[r];
-                if (c.sum_b != nullptr) e_sb = (float)c.sum_b[r];
-            }
+        // threads that finish the rows do not start a memory round trip after the last barrier.  All six requests go out
+        // back to back, whatever terms the call has (a term that does not exist reads the output row instead and is
+        // dropped later), and nothing is done with the values until the epilogue: with one conditional load per term the
+        // compiler waited for each of them in turn, three or four dependent memory round trips in front of the first
+        // weight tile of the wave that finishes the rows - it saw every event of the pass several microseconds after the
+        // other waves, and the whole workgroup ended that much later.
+        const int et = (int)threadIdx.x;
+        const bool finisher = et < b1 - b0;
+        half_t h_b1, h_b2, h_x0, h_x1, h_sa, h_sb;      // (only read by the lanes that loaded them)
+        if (first_lane(et >> 6) == 0) {     // the wave that holds the finishing lanes (a scalar branch)
+            const int r = finisher ? b0 + et : b0;
+            const half_t* any = c.out + r;
+            h_b1 = *(c.bias1 ? c.bias1 + r : any);
+            h_b2 = *(c.bias2 ? c.bias2 + r : any);
+            h_x0 = *(c.base0 ? c.base0 + r : any);
+            h_x1 = *(c.base1 ? c.base1 + r : any);
+            h_sa = *((c.sum_b != nullptr || c.add_sum) ? c.sum_a + r : any);
+            h_sb = *(c.sum_b ? c.sum_b + r : any);
+            __builtin_amdgcn_sched_barrier(0);
         }
         if (streamer && c.K2 > 0) down_phases<CPD, 0>(c, ks, lane, b0, b1, sh, first, down_ready);
         if (o_index >= 0 && c.K1 > 0) {
@@ -1417,9 +1451,9 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
         }
         first = false;
         __syncthreads();
-        const int t = threadIdx.x;
-        if (t < b1 - b0) {
-            const int r = b0 + t;
+        if (finisher) {
+            const int t = et, r = b0 + et;
+            const float e_b1 = (float)h_b1, e_b2 = (float)h_b2, e_x0 = (float)h_x0, e_x1 = (float)h_x1, e_sa = (float)h_sa, e_sb = (float)h_sb;
             float v = 0.f;
             if (c.K2 > 0) {
 #pragma unroll

@@ -9,6 +9,7 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -61,14 +62,16 @@ __device__ __forceinline__ void qkv_rows(const LayerParams& p, const half2_t (&x
 template <int NCH, bool EX>
 __device__ __forceinline__ void qkv_prefetch(const LayerParams& p, const RowWalk& rw, int lane,
                                              RowTile<NCH, StageARpi<NCH>::value>& pre) {
-    if (rw.ntiles > 0) load_row_tile<NCH, StageARpi<NCH>::value, EX>(pre, p.w_qkv, p.H, rw.first, rw.sit, rw.end, lane);
+    prefetch_row_tile<NCH, StageARpi<NCH>::value, EX>(pre, p.w_qkv, p.H, rw.first, rw.sit, rw.end, rw.ntiles, lane);
 }
 
 // MLP-up rows of one streaming wave (tiles of kUpRpi adjacent rows); result = gelu(dot + bias) as fp16.
 // up_prefetch requests the first tile (before something slow: a LayerNorm, an event), up_rows consumes it.
 template <int NCH, bool EX>
 __device__ __forceinline__ void up_prefetch(const LayerParams& p, const RowWalk& rw, int lane, RowTile<NCH, kUpRpi>& pre) {
-    if (rw.ntiles > 0) load_row_tile<NCH, kUpRpi, EX>(pre, p.w_up, p.H, rw.first, rw.sit, rw.end, lane);
+    // (a layer without MLP has no W_up at all: its waves, which have no tiles, request row 0 of W_qkv instead)
+    prefetch_row_tile<NCH, kUpRpi, EX>(pre, p.w_up != nullptr ? p.w_up : p.w_qkv, p.H, rw.first, rw.sit, rw.end,
+                                       p.w_up != nullptr ? rw.ntiles : 0, lane);
 }
 template <int NCH, bool EX>
 __device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], const RowWalk& rw, int lane,
@@ -213,7 +216,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_up(LayerParams p) {
     ln_coop_load<NCH, kStreamers, false>(own, norm_spec(p), wave, lane);
     __builtin_amdgcn_sched_barrier(0);   // the norm inputs go out first
     RowTile<NCH, 2> t0;
-    if (count > 0) load_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, lane);
+    prefetch_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, count, lane);
     ln_coop_finish<NCH, kStreamers, false>(own, norm_spec(p), lns, wave, lane);
     half2_t xr[NCH][4];
     ln_fetch<NCH>(lns, 0, lane, xr);
@@ -257,7 +260,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
     ln_coop_load<NCH, kStreamers, false>(own, norm_spec(p), wave, lane);
     __builtin_amdgcn_sched_barrier(0);   // the norm inputs go out first
     RowTile<NCH, 2> t0;
-    if (count > 0) load_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, lane);
+    prefetch_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, count, lane);
     ln_coop_finish<NCH, kStreamers, false>(own, norm_spec(p), lns, wave, lane);
     const int tag = first_lane(gen) + 1;
     half2_t xr[NCH][4];
@@ -272,7 +275,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
             });
         if (g + 1 < kUpPhases) {
             share(g + 1, first, count);
-            if (count > 0) load_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, lane);     // in flight across the event
+            prefetch_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, count, lane);     // in flight across the event
         }
         event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &arrived[g], kStreamers, tag);
     }
@@ -357,9 +360,10 @@ struct FusedLds {
     float park_attn[kStreamers][kParkRows];   // QKV rows of the attention waves
 };
 
-// One layer; `gen` is the launch generation read at the start of the launch.
+// One layer; `gen_word` is the word the launch tag derives from (the generation of the workspace, or the caller's step
+// counter), requested at the start of the launch.
 template <int NCH, int CPD, bool EX, bool BYX>
-__device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, FusedLds<NCH>& lds) {
+__device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, FusedLds<NCH>& lds) {
     FusedShared& q = lds.q;
     StageCShared& shc = lds.shc;
     LnShared<NCH>& lns = lds.lns;
@@ -369,6 +373,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
     const int G = gridDim.x, b = blockIdx.x;
     const int nsw = G * kStreamers;                 // streaming waves in the grid
     const StatusSink status = status_sink(p);
+    const int seq_requested = seq_len_request(p);     // on its way before anything else
     if (threadIdx.x <= kUpPhases) q.arrived[threadIdx.x] = 0;
     __syncthreads();
     trace_mark(p, 0);
@@ -391,20 +396,31 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
     const int qkv_arrivals = qkv8 ? kFusedWaves : kStreamers;
     const int hw = wave - kStreamers;
     RowTile<NCH, RPIA> t0;
-    {
+    // The norm, with or without a first weight tile requested behind its inputs.  The two cases are two copies of the code,
+    // not one copy with a branch around the tile's loads: behind such a branch the compiler's wait for the norm's inputs
+    // waits for the tile as well (it counts the loads in flight by the shorter path), and the norm of the whole workgroup
+    // then starts when the slowest wave's tile has arrived instead of when the input row has.
+    auto norm_phase = [&](auto with_tile) {
         LnOwn<NCH, kFusedWaves> own;
         ln_coop_load<NCH, kFusedWaves, true>(own, norm_spec(p), wave, lane);
         __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
-        if (qkv8 || wave < kStreamers) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
+        if constexpr (decltype(with_tile)::value) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
         trace_mark(p, 14);
 #ifdef CFPP_TRACE
         trace_value(p, 15, wall_clock64() + (long long)(own.rx[0].x & 0u));     // the wave's chunk of the input row has arrived
 #endif
         ln_coop_finish<NCH, kFusedWaves, true>(own, norm_spec(p), lns, wave, lane);
-    }
-    const int tag = first_lane(gen) + 1;
-    const SeqLen sl = load_seq_len(p);
-    const int nsplit = effective_split(p, sl.S), per_head = items_per_head(nsplit);
+    };
+    if (qkv8 || wave < kStreamers) norm_phase(std::true_type{});
+    else norm_phase(std::false_type{});
+    trace_mark(p, 1);
+    // The launch tag and the sequence length were requested at the top of the kernel.  They are looked at (`resolve`)
+    // only once a wave has used up its first weight tile: every load of a wave returns in order, so by then they are
+    // there for free, whereas waiting for them right here would also wait for the tile in flight, with the request for
+    // the next tile still to come - a memory round trip with nothing in flight at the start of every wave's rows.
+    int tag = 0, nsplit = 1, per_head = 2, item_lo = 0, item_step = 1, nitems = 0, head_lo = 0, attn_count = 0;
+    SeqLen sl{0, true};
+    bool by_xcd = false, agent_up = false;
     // Which (head, split) items the attention waves of this workgroup take.  Normally item b + hw G.  When a head's slice
     // of a cache row is not a whole number of 128-byte memory lines (80-dim heads: 160 bytes), neighbouring heads share
     // lines, and each of the eight chiplets, with its own L2, would fetch a shared line again: the heads are then dealt
@@ -414,19 +430,25 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
     // at 512, but +0.7 % at 1536 and +1.5 % at 4096).
     // BYX is the host's part of the condition (head size, head count and grid; a template flag, so that layers whose
     // heads are whole lines carry none of this).
-    const bool by_xcd = BYX && (long long)sl.S * (p.heads / kXcds) * p.D * 4 <= kXcdGroupBytes;
-    const int item_lo = by_xcd ? b / kXcds : b, item_step = by_xcd ? G / kXcds : G;
-    const int nitems = (by_xcd ? p.heads / kXcds : p.heads) * per_head;        // of this workgroup's chiplet / of the layer
-    const int head_lo = by_xcd ? (b % kXcds) * (p.heads / kXcds) : 0;
-    const int attn_count = nitems > item_lo ? (nitems - item_lo + item_step - 1) / item_step : 0;
-    trace_mark(p, 1);
     // Counting an arrival device-wide is two dependent atomic round trips for the wave that does it, and a
     // streaming wave that stops for them falls behind its workgroup (and then is the last one again at the next
     // event).  When the workgroup has an attention wave without an item (fewer than four items), the streaming
     // waves only drain their stores and count themselves in LDS at the MLP-up events, and that idle wave carries
     // the count to the device-wide counters.  (Not at the QKV event: the attention waves wait for that one, and
     // an arrival that goes through another wave reaches them later.)
-    const bool agent_up = p.arrival_agents && attn_count < kStreamers;
+    auto resolve = [&]() {
+        tag = first_lane(gen_word) * (p.tag_src != nullptr ? p.tag_mul : 1) + (p.tag_src != nullptr ? p.tag_add : 0) + 1;
+        sl = seq_len_check(p, first_lane(seq_requested));
+        nsplit = effective_split(p, sl.S);
+        per_head = items_per_head(nsplit);
+        by_xcd = BYX && (long long)sl.S * (p.heads / kXcds) * p.D * 4 <= kXcdGroupBytes;
+        item_lo = by_xcd ? b / kXcds : b;
+        item_step = by_xcd ? G / kXcds : G;
+        nitems = (by_xcd ? p.heads / kXcds : p.heads) * per_head;        // of this workgroup's chiplet / of the layer
+        head_lo = by_xcd ? (b % kXcds) * (p.heads / kXcds) : 0;
+        attn_count = nitems > item_lo ? (nitems - item_lo + item_step - 1) / item_step : 0;
+        agent_up = p.arrival_agents && attn_count < kStreamers;
+    };
     auto stream_arrive = [&](int event, int* lds_ctr, bool agent) {
         if (agent) {
             drain_memory_ops();
@@ -453,6 +475,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
         half2_t xr[NCH][4];   // ln1(x) for the QKV rows, then ln2(x) for the MLP-up rows
         ln_fetch<NCH>(lns, 0, lane, xr);
         qkv_rows<NCH, EX>(p, xr, qw, lane, t0, spark);
+        resolve();
         // the MLP-up tiles of a phase are handed out dynamically within the team; the first tile of the next
         // pass is requested before the event that ends this one, so the wave is not left without loads in flight
         // (only when a wave can expect four tiles or more per phase: with fewer, the static shares are
@@ -506,9 +529,12 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen, Fused
             // further back
             __builtin_amdgcn_s_setprio(2);
             qkv_rows<NCH, EX>(p, xq, qw, lane, t0, hpark);
+            resolve();
             event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
             __builtin_amdgcn_s_setprio(0);
             trace_mark(p, 2);
+        } else {
+            resolve();
         }
         if (hw < attn_count) {
             AttnItem it;
@@ -552,10 +578,9 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     // the flag value of this launch is gen + 1: requested first, needed at the first event.  It comes from the
     // generation the previous launch on this workspace published, or from a counter that the caller advances
     // between launches (a whole-model step: step counter x layers + layer), which saves the publishing.
-    // (a vector load, not waited for until the first event needs the tag)
-    const int gen = counter_peek(p.tag_src != nullptr ? p.tag_src : p.bar + kBarGen) * (p.tag_src != nullptr ? p.tag_mul : 1) +
-                    (p.tag_src != nullptr ? p.tag_add : 0);
-    fused_layer<NCH, CPD, EX, BYX>(p, gen, lds);
+    // (a vector load; nothing looks at the value until the wave has used up its first weight tile)
+    const int gen_word = counter_peek(p.tag_src != nullptr ? p.tag_src : p.bar + kBarGen);
+    fused_layer<NCH, CPD, EX, BYX>(p, gen_word, lds);
 }
 
 // ---- whole-model helpers -----------------------------------------------------------------------
@@ -590,7 +615,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __res
     ln_coop_load<NCH, NWV, false>(own, ns, wave, lane);
     __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
     RowTile<NCH, RPIA> t0;
-    if (rw.ntiles > 0) load_row_tile<NCH, RPIA, EX>(t0, W, H, rw.first, rw.sit, rw.end, lane);
+    prefetch_row_tile<NCH, RPIA, EX>(t0, W, H, rw.first, rw.sit, rw.end, rw.ntiles, lane);
     ln_coop_finish<NCH, NWV, false>(own, ns, lns, wave, lane);
     half2_t x1[NCH][4];
     ln_fetch<NCH>(lns, 0, lane, x1);
