@@ -120,6 +120,14 @@ def build_ext():
     return EXT
 
 
+def build_stream_probe(out=os.path.join(PKG, "stream_probe_bin")):
+    """The bare read probes (csrc/stream_probe.hip) as an executable next to this file; a measurement tool."""
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    _run([hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          "-Wno-unused-command-line-argument", os.path.join(CSRC, "stream_probe.hip"), "-o", out])
+    return out
+
+
 def build_all():
     build_lib()
     build_ext()
@@ -130,10 +138,13 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--trace-lib", metavar="PATH",
                     help="only build a profiling variant of the HIP library (-DCFPP_TRACE) at PATH (not the product library's path)")
+    ap.add_argument("--stream-probe", action="store_true", help="only build the bare read probes (stream_probe.py runs them)")
     ap.add_argument("--resource-report", action="store_true",
                     help="only print registers, scratch, LDS and occupancy of every kernel (compiler remarks)")
     a = ap.parse_args()
-    if a.resource_report:
+    if a.stream_probe:
+        build_stream_probe()
+    elif a.resource_report:
         print(resource_report())
     elif a.trace_lib:
         build_lib(trace=True, out=a.trace_lib)
