@@ -903,20 +903,30 @@ struct StageARpi { static constexpr int value = (16 / NCH) > 0 ? (16 / NCH) : 1;
 struct RopeCoeffs { float c[8], sg[8]; };
 template <bool PAIRS = false>
 __device__ __forceinline__ void rope_coeffs(int d0, int rot, const float* __restrict__ cs, const float* __restrict__ sn,
-                                            bool act, bool half_table, RopeCoeffs& rc) {
+                                            bool act, bool half_table, const float* __restrict__ readable, RopeCoeffs& rc) {
+    // Every lane loads all sixteen values, whether it needs them or not (a lane or dim without rotation reads entry 0,
+    // a geometry without rotation reads `readable`, any readable device memory): loads under a condition would each
+    // be waited for where their branch ends, one memory round trip after the other.
     const int hr = rot >> 1;
+    const float* __restrict__ c0 = rot > 0 ? cs : readable;
+    const float* __restrict__ s0 = rot > 0 ? sn : readable;
+    float cv[8], sv[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int d = d0 + j;
         const bool rotd = act && d < rot;
-        if (PAIRS) {
-            rc.c[j] = rotd ? cs[d] : 1.f;
-            rc.sg[j] = rotd ? ((d & 1) ? sn[d] : -sn[d]) : 0.f;
-        } else {
-            const int t = (half_table && d >= hr) ? d - hr : d;
-            rc.c[j] = rotd ? cs[t] : 1.f;
-            rc.sg[j] = rotd ? (d < hr ? -sn[t] : sn[t]) : 0.f;
-        }
+        const int t = PAIRS ? d : ((half_table && d >= hr) ? d - hr : d);
+        const int ti = rotd ? t : 0;
+        cv[j] = c0[ti];
+        sv[j] = s0[ti];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int d = d0 + j;
+        const bool rotd = act && d < rot;
+        rc.c[j] = rotd ? cv[j] : 1.f;
+        if (PAIRS) rc.sg[j] = rotd ? ((d & 1) ? sv[j] : -sv[j]) : 0.f;
+        else rc.sg[j] = rotd ? (d < hr ? -sv[j] : sv[j]) : 0.f;
     }
 }
 // The raw values of a lane's eight dims and of their rotation partners: rope_request issues the loads, rope_finish
@@ -974,12 +984,32 @@ __device__ __forceinline__ void raw_load8(const float* __restrict__ v, int d0, b
 constexpr int kAttnT = 8;
 constexpr int kAttnTileRows = 4 * kAttnT;
 struct KvTile { u32x4 k[kAttnT], v[kAttnT]; };
+struct KvRows { int r[kAttnT]; };     // paged caches: the cache rows of a tile's kAttnT rows of this lane's group
 struct AttnItem {
     int head, sp, nsplit, S, begin, end, ntiles;
     bool append_ok;     // the sequence length was valid: split 0 may append the new row
     KvTile t0, t1;
+    KvRows r0, r1;      // PAGED: page-table entries of the tiles that t0 / t1 take next
     RopeCoeffs rc;
 };
+// PAGED: the page-table entries of tile i (rows past the end repeat the last row, tiles past the end as well).  They
+// are requested two tiles before the K/V rows they address, so that a tile costs one memory round trip, not two.
+__device__ __forceinline__ void attn_request_rows(const LayerParams& p, const AttnItem& it, KvRows& rows, int i, int lane) {
+    const int r = it.begin + i * kAttnTileRows + (lane >> 4);
+#pragma unroll
+    for (int t = 0; t < kAttnT; ++t) rows.r[t] = p.kv_rows[min(r + t * 4, it.end - 1)];
+}
+__device__ __forceinline__ void attn_load_tile_rows(const LayerParams& p, const AttnItem& it, KvTile& kv, const KvRows& rows, int lane) {
+    const int sub = lane & 15;
+    const int d0 = sub * 8 < p.D ? sub * 8 : 0;
+    const half_t* __restrict__ kc = p.k_cache + (size_t)it.head * p.D + d0;
+    const half_t* __restrict__ vc = p.v_cache + (size_t)it.head * p.D + d0;
+#pragma unroll
+    for (int t = 0; t < kAttnT; ++t) {
+        kv.k[t] = ld16(kc + (size_t)rows.r[t] * p.H);
+        kv.v[t] = ld16(vc + (size_t)rows.r[t] * p.H);
+    }
+}
 // tile i of the item; rows past the end re-read the last row (masked when used): no conditional loads
 // PAGED: rows go through p.kv_rows
 template <bool PAGED = false>
@@ -1005,13 +1035,25 @@ __device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it
     it.begin = sp < nsplit ? sp * chunk : S;          // item nsplit (if it exists) is the new token: no cache rows
     it.end = (it.begin + chunk < S) ? it.begin + chunk : S;
     it.ntiles = it.begin < it.end ? (it.end - it.begin + kAttnTileRows - 1) / kAttnTileRows : 0;
-    if (it.ntiles > 0) attn_load_tile<PAGED>(p, it, it.t0, 0, lane);
-    if (it.ntiles > 1) attn_load_tile<PAGED>(p, it, it.t1, 1, lane);
+    // the coefficients first: what waits for them then does not wait for the tiles as well
     const int sub = lane & 15;
     const bool act = sub * 8 < p.D;
     const float* __restrict__ cs = p.cos + (size_t)S * p.rope_stride;   // stride 0: the row is the position
     const float* __restrict__ sn = p.sin + (size_t)S * p.rope_stride;
-    rope_coeffs<PAIRS>(act ? sub * 8 : 0, p.rot, cs, sn, act, p.rope_half_table != 0, it.rc);
+    rope_coeffs<PAIRS>(act ? sub * 8 : 0, p.rot, cs, sn, act, p.rope_half_table != 0, p.qkv_raw, it.rc);
+    if (PAGED) {
+        if (it.ntiles > 0) {
+            attn_request_rows(p, it, it.r0, 0, lane);
+            attn_request_rows(p, it, it.r1, 1, lane);
+            attn_load_tile_rows(p, it, it.t0, it.r0, lane);
+            attn_load_tile_rows(p, it, it.t1, it.r1, lane);
+            attn_request_rows(p, it, it.r0, 2, lane);
+            attn_request_rows(p, it, it.r1, 3, lane);
+        }
+    } else {
+        if (it.ntiles > 0) attn_load_tile<PAGED>(p, it, it.t0, 0, lane);
+        if (it.ntiles > 1) attn_load_tile<PAGED>(p, it, it.t1, 1, lane);
+    }
 }
 
 // nwg_to_signal > 0 (fused kernel): a completed head counts towards the kBarHeads event of that many workgroups.
@@ -1114,18 +1156,20 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
             m = mt;
         };
         if (PAGED) {
-            // items of a batched launch can be long: keep two tiles in flight all the way
+            // Items of a batched launch can be long: two tiles in flight all the way, and the page-table entries of the
+            // two after them.  No branch in the loop (a tile past the end repeats the item's last row and is masked
+            // where it is used), so that no wait covers more than the tile it is for.
             for (int i = 0; i < it.ntiles; i += 2) {
                 process(it.t0, i);
                 __builtin_amdgcn_sched_barrier(0);
-                if (i + 2 < it.ntiles) attn_load_tile<PAGED>(p, it, it.t0, i + 2, lane);
+                attn_load_tile_rows(p, it, it.t0, it.r0, lane);
+                attn_request_rows(p, it, it.r0, i + 4, lane);
                 __builtin_amdgcn_sched_barrier(0);
-                if (i + 1 < it.ntiles) {
-                    process(it.t1, i + 1);
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (i + 3 < it.ntiles) attn_load_tile<PAGED>(p, it, it.t1, i + 3, lane);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+                process(it.t1, i + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                attn_load_tile_rows(p, it, it.t1, it.r1, lane);
+                attn_request_rows(p, it, it.r1, i + 5, lane);
+                __builtin_amdgcn_sched_barrier(0);
             }
         } else {
             if (it.ntiles > 0) process(it.t0, 0);
