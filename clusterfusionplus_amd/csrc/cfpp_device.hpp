@@ -541,7 +541,20 @@ __device__ __forceinline__ void ln_fetch(const LnShared<NCH>& sh, int which, int
 template <int NCH, int RPI>
 struct RowTile {
     u32x4 w[RPI][NCH];
+    half_t bias;     // of the row that this lane stores after the wave's first segment of rows, requested with the first tile
+                     // (row_bias_request; the functions that have no use for it leave it alone)
 };
+
+// The value that lane `lane` adds to the row it stores when a wave's parked rows are written out: requested together with
+// the wave's first tile, because at the end of the rows it would be one more memory round trip, behind the tile already
+// requested for the next pass, between the wave's last product and the event that other waves wait for.  `row` is clamped
+// into [0, end); a null `b` reads `readable` instead (any readable device memory; the caller ignores the value).
+__device__ __forceinline__ half_t row_bias_request(const half_t* __restrict__ b, const void* readable, int row, int end) {
+    const half_t* __restrict__ src = b != nullptr ? b : reinterpret_cast<const half_t*>(readable);
+    int r = row < end ? row : end - 1;
+    r = r > 0 ? r : 0;
+    return src[r];
+}
 
 // Issue the loads of rows r, r+stride, ... (RPI of them; rows >= nrows repeat row r).  EXACT: K ==
 // NCH*512, every lane load is in range; otherwise out-of-range lane loads are redirected to column 0
@@ -780,16 +793,40 @@ __device__ __forceinline__ void finish_refill_team_tile(RowTile<NCH, RPI>& t, co
 // team_prefetch requests the wave's first ticket and its two static tiles (before something slow: the
 // LayerNorm, an event); gemv_team consumes them.  flush(park) runs outside the streaming loop, when the
 // park is full and at the end; parked value k belongs to row park.row[k].
+constexpr int kTeamBiasRegs = 4;       // a team's rows of a pass whose biases its waves hold: 64 per register
 template <int NCH, int RPI>
 struct TeamTiles {
     RowTile<NCH, RPI> a, b;
     int req;
+    half_t bias[kTeamBiasRegs];        // lane l, register k: the bias of row tm.row0 + 64 k + l (team_bias_held)
 };
+// A wave cannot know which rows of the team's range it will get, so it requests the biases of all of them (when the
+// range is short enough), one row per lane and register, and picks its rows' values from the lanes that hold them when
+// it stores them (team_bias).  For the reason see row_bias_request.
+template <int RPI>
+__device__ __forceinline__ bool team_bias_held(const TileTeam& tm) { return tm.ntiles * RPI <= 64 * kTeamBiasRegs; }
+template <int NCH, int RPI>
+__device__ __forceinline__ float team_bias(const TileTeam& tm, const TeamTiles<NCH, RPI>& tt, const half_t* __restrict__ b, int row,
+                                           bool valid) {
+    if (team_bias_held<RPI>(tm)) {          // the same for the whole wave
+        const int rel = valid ? row - tm.row0 : 0;
+        float v = 0.f;
+#pragma unroll
+        for (int k = 0; k < kTeamBiasRegs; ++k) {
+            const int got = __builtin_amdgcn_ds_bpermute((rel & 63) << 2, (int)__builtin_bit_cast(unsigned short, tt.bias[k]));
+            if ((rel >> 6) == k) v = (float)__builtin_bit_cast(half_t, (unsigned short)got);
+        }
+        return v;
+    }
+    return valid ? (float)b[row] : 0.f;
+}
 template <int NCH, int RPI, bool EXACT>
 __device__ __forceinline__ void team_prefetch(const half_t* __restrict__ W, int K, const TileTeam& tm, int lane,
-                                              TeamTiles<NCH, RPI>& tt) {
+                                              TeamTiles<NCH, RPI>& tt, const half_t* __restrict__ bias) {
     tt.req = ticket_request(tm.counter, lane);
     if (tm.j < tm.ntiles) load_row_tile<NCH, RPI, EXACT>(tt.a, W, K, tm.row0 + tm.j * RPI, 1, tm.end, lane);
+#pragma unroll
+    for (int k = 0; k < kTeamBiasRegs; ++k) tt.bias[k] = row_bias_request(bias, W, tm.row0 + 64 * k + lane, tm.end);
 }
 template <int NCH, int RPI, bool EXACT, bool ROLL = false, class Flush>
 __device__ __forceinline__ void gemv_team(const half_t* __restrict__ W, int K, const TileTeam& tm, const half2_t (&x)[NCH][4],

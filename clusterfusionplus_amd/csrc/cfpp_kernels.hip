@@ -50,12 +50,15 @@ __device__ __forceinline__ void qkv_rows(const LayerParams& p, const half2_t (&x
                                          RowTile<NCH, StageARpi<NCH>::value>& pre, RowPark& park) {
     constexpr int RPI = StageARpi<NCH>::value;
     const int first = rw.first, step = rw.step;
+    const half_t bias0 = pre.bias;
     gemv_tiles<NCH, RPI, EX, RollTiles<NCH>::value>(
         p.w_qkv, p.H, rw.end, rw.sit, rw.ntiles, [=](int t) { return first + t * step; }, x1, lane, pre, park,
         [&](const RowPark& pk, int k0) {
             if (lane < pk.n) {
                 const int row = walk_row<RPI>(rw, k0 + lane);
-                st_agent(p.qkv_raw + row, pk.slot[lane] + (p.b_qkv ? (float)p.b_qkv[row] : 0.f));
+                float bias = (float)bias0;                       // the first segment's was requested with the first tile
+                if (k0 != 0 && p.b_qkv != nullptr) bias = (float)p.b_qkv[row];
+                st_agent(p.qkv_raw + row, pk.slot[lane] + (p.b_qkv != nullptr ? bias : 0.f));
             }
         });
 }
@@ -63,6 +66,7 @@ template <int NCH, bool EX>
 __device__ __forceinline__ void qkv_prefetch(const LayerParams& p, const RowWalk& rw, int lane,
                                              RowTile<NCH, StageARpi<NCH>::value>& pre) {
     prefetch_row_tile<NCH, StageARpi<NCH>::value, EX>(pre, p.w_qkv, p.H, rw.first, rw.sit, rw.end, rw.ntiles, lane);
+    pre.bias = row_bias_request(p.b_qkv, p.w_qkv, walk_row<StageARpi<NCH>::value>(rw, lane), rw.end);
 }
 
 // MLP-up rows of one streaming wave (tiles of kUpRpi adjacent rows); result = gelu(dot + bias) as fp16.
@@ -72,17 +76,21 @@ __device__ __forceinline__ void up_prefetch(const LayerParams& p, const RowWalk&
     // (a layer without MLP has no W_up at all: its waves, which have no tiles, request row 0 of W_qkv instead)
     prefetch_row_tile<NCH, kUpRpi, EX>(pre, p.w_up != nullptr ? p.w_up : p.w_qkv, p.H, rw.first, rw.sit, rw.end,
                                        p.w_up != nullptr ? rw.ntiles : 0, lane);
+    pre.bias = row_bias_request(p.b_up, p.w_qkv, walk_row<kUpRpi>(rw, lane), rw.end);
 }
 template <int NCH, bool EX>
 __device__ __forceinline__ void up_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], const RowWalk& rw, int lane,
                                         RowTile<NCH, kUpRpi>& pre, RowPark& park) {
     const int first = rw.first, step = rw.step;
+    const half_t bias0 = pre.bias;
     gemv_tiles<NCH, kUpRpi, EX, RollTiles<NCH>::value>(
         p.w_up, p.H, rw.end, rw.sit, rw.ntiles, [=](int t) { return first + t * step; }, x2, lane, pre, park,
         [&](const RowPark& pk, int k0) {
             if (lane < pk.n) {
                 const int row = walk_row<kUpRpi>(rw, k0 + lane);
-                st_agent(p.inter + row, (half_t)gelu_tanh(pk.slot[lane] + (float)p.b_up[row]));
+                float bias = (float)bias0;                       // the first segment's was requested with the first tile
+                if (k0 != 0) bias = (float)p.b_up[row];
+                st_agent(p.inter + row, (half_t)gelu_tanh(pk.slot[lane] + bias));
             }
         });
 }
@@ -104,26 +112,14 @@ __device__ __forceinline__ TileTeam make_team(const LayerParams& p, int pass, in
     tm.end = hi;
     return tm;
 }
-// QKV rows: result = dot + bias as raw fp32
-template <int NCH, bool EX>
-__device__ __forceinline__ void qkv_team_rows(const LayerParams& p, const half2_t (&x1)[NCH][4], const TileTeam& tm, int lane,
-                                              TeamTiles<NCH, StageARpi<NCH>::value>& tt, RowParkIds& park) {
-    gemv_team<NCH, StageARpi<NCH>::value, EX>(p.w_qkv, p.H, tm, x1, lane, tt, park, [&](const RowParkIds& pk) {
-        if (lane < pk.n) {
-            const int row = pk.row[lane];
-            if (row >= 0) st_agent(p.qkv_raw + row, pk.slot[lane] + (p.b_qkv ? (float)p.b_qkv[row] : 0.f));
-        }
-    });
-}
 // MLP-up rows: result = gelu(dot + bias) as fp16
 template <int NCH, bool EX>
 __device__ __forceinline__ void up_team_rows(const LayerParams& p, const half2_t (&x2)[NCH][4], const TileTeam& tm, int lane,
                                              TeamTiles<NCH, kUpRpi>& tt, RowParkIds& park) {
     gemv_team<NCH, kUpRpi, EX, RollTiles<NCH>::value>(p.w_up, p.H, tm, x2, lane, tt, park, [&](const RowParkIds& pk) {
-        if (lane < pk.n) {
-            const int row = pk.row[lane];
-            if (row >= 0) st_agent(p.inter + row, (half_t)gelu_tanh(pk.slot[lane] + (float)p.b_up[row]));
-        }
+        const int row = lane < pk.n ? pk.row[lane] : -1;
+        const float bias = team_bias<NCH, kUpRpi>(tm, tt, p.b_up, row, row >= 0);     // by all lanes: values cross lanes
+        if (row >= 0) st_agent(p.inter + row, (half_t)gelu_tanh(pk.slot[lane] + bias));
     });
 }
 
@@ -273,11 +269,13 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
             [&](const RowPark& pk, int k0) {
                 if (2 * lane + 1 < pk.n) st_agent(p.inter + f + k0 / 2 + lane, (half_t)(silu(pk.slot[2 * lane]) * pk.slot[2 * lane + 1]));
             });
+        // counted in before the next pass's first tile is requested: the count waits for this wave's stores, and would
+        // wait for that tile as well
+        event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &arrived[g], kStreamers, tag);
         if (g + 1 < kUpPhases) {
             share(g + 1, first, count);
-            prefetch_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, count, lane);     // in flight across the event
+            prefetch_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, count, lane);
         }
-        event_arrive(p.bar, p.grp, p.mbox, kBarUp + g, G, &arrived[g], kStreamers, tag);
     }
     const StageC c = make_stage_c(p);
     stage_c_rows<NCH, CPD>(c, b, G, shc, true, wave, wave, kStreamers, lane,
@@ -395,7 +393,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
                                              wave < kStreamers ? 3 * p.H : 0);
     const int qkv_arrivals = qkv8 ? kFusedWaves : kStreamers;
     const int hw = wave - kStreamers;
-    RowTile<NCH, RPIA> t0;
+    RowTile<NCH, StageARpi<NCH>::value> t0;
     // The norm, with or without a first weight tile requested behind its inputs.  The two cases are two copies of the code,
     // not one copy with a branch around the tile's loads: behind such a branch the compiler's wait for the norm's inputs
     // waits for the tile as well (it counts the loads in flight by the shorter path), and the norm of the whole workgroup
@@ -476,16 +474,19 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
         ln_fetch<NCH>(lns, 0, lane, xr);
         qkv_rows<NCH, EX>(p, xr, qw, lane, t0, spark);
         resolve();
-        // the MLP-up tiles of a phase are handed out dynamically within the team; the first tile of the next
-        // pass is requested before the event that ends this one, so the wave is not left without loads in flight
-        // (only when a wave can expect four tiles or more per phase: with fewer, the static shares are
-        // already as fine as the tickets, and the ticket round trips cost more than they balance)
+        // the MLP-up tiles of a phase are handed out dynamically within the team (only when a wave can expect four
+        // tiles or more per phase: with fewer, the static shares are already as fine as the tickets, and the ticket
+        // round trips cost more than they balance)
         TileTeam utm = make_team<kUpRpi>(p, 1, 0, up_phase_rows(CPD, 0, p.F), b, G, wave);
         const bool dynamic = utm.ntiles >= 4 * utm.nw;
+        // A wave counts itself in for an event before it requests the first tile of its next pass: the count has to wait
+        // for the wave's stores, and that wait would be for the requested tile as well (one counter covers both).  The
+        // exception are the MLP-up phases with shared tiles, where the request goes first: there the tile in flight
+        // at the hand-over is worth more than the earlier event (both orders measured, on both models).
         if (dynamic) {
             TeamTiles<NCH, kUpRpi> ut;
-            team_prefetch<NCH, kUpRpi, EX>(p.w_up, p.H, utm, lane, ut);
             event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
+            team_prefetch<NCH, kUpRpi, EX>(p.w_up, p.H, utm, lane, ut, p.b_up);
             trace_mark(p, 2);
             ln_fetch<NCH>(lns, 1, lane, xr);
 #pragma unroll
@@ -493,7 +494,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
                 up_team_rows<NCH, EX>(p, xr, utm, lane, ut, park);
                 if (g + 1 < kUpPhases) {
                     utm = make_team<kUpRpi>(p, 2 + g, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F), b, G, wave);
-                    team_prefetch<NCH, kUpRpi, EX>(p.w_up, p.H, utm, lane, ut);
+                    team_prefetch<NCH, kUpRpi, EX>(p.w_up, p.H, utm, lane, ut, p.b_up);
                 }
                 stream_arrive(kBarUp + g, &q.arrived[1 + g], agent_up);
                 trace_mark(p, g == kUpPhases - 1 ? 5 : 12);
@@ -501,18 +502,18 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
         } else {
             RowTile<NCH, kUpRpi> u0;
             RowWalk uw = row_walk<kUpRpi>(b * kStreamers + wave, nsw, 0, up_phase_rows(CPD, 0, p.F));
-            up_prefetch<NCH, EX>(p, uw, lane, u0);
             event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
+            up_prefetch<NCH, EX>(p, uw, lane, u0);
             trace_mark(p, 2);
             ln_fetch<NCH>(lns, 1, lane, xr);
 #pragma unroll
             for (int g = 0; g < kUpPhases; ++g) {
                 up_rows<NCH, EX>(p, xr, uw, lane, u0, spark);
+                stream_arrive(kBarUp + g, &q.arrived[1 + g], agent_up);
                 if (g + 1 < kUpPhases) {
                     uw = row_walk<kUpRpi>(b * kStreamers + wave, nsw, up_phase_rows(CPD, g, p.F), up_phase_rows(CPD, g + 1, p.F));
                     up_prefetch<NCH, EX>(p, uw, lane, u0);
                 }
-                stream_arrive(kBarUp + g, &q.arrived[1 + g], agent_up);
                 trace_mark(p, g == kUpPhases - 1 ? 5 : 12);
             }
         }
