@@ -1094,8 +1094,12 @@ __device__ __forceinline__ void attn_prefetch(const LayerParams& p, AttnItem& it
 }
 
 // nwg_to_signal > 0 (fused kernel): a completed head counts towards the kBarHeads event of that many workgroups.
+// The partial result of an item whose head is merged inside the workgroup (AttnLdsPart, one per wave): the dims of lane
+// group 0 after the merge of the wave's four groups, and the softmax state.
+struct AttnLdsPart { float acc[128]; float m, l; };
 template <bool PAGED = false, bool PAIRS = false>
-__device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& it, int lane, int nwg_to_signal, int tag) {
+__device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& it, int lane, int nwg_to_signal, int tag,
+                                               AttnLdsPart* lds_part = nullptr) {
     const int grp = lane >> 4, sub = lane & 15;
     const int D = p.D, H = p.H;
     const int head = it.head, sp = it.sp, nsplit = it.nsplit, S = it.S, end = it.end;
@@ -1238,6 +1242,15 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
             acc[j] = a;
         }
         m = mw;
+    }
+    if (lds_part != nullptr) {
+        // the splits of this head run in this workgroup: the partial goes to LDS, the caller merges behind a barrier
+        if (grp == 0 && act) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) lds_part->acc[d0 + j] = acc[j];
+            if (sub == 0) { lds_part->m = m; lds_part->l = l; }
+        }
+        return;
     }
     // publish the partial of this (head, split)
     const size_t item = (size_t)head * kMaxSplit + sp;

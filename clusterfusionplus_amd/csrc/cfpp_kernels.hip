@@ -983,25 +983,33 @@ __global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
         u32x4 w[16], x0[16];
         request(w, b0);
         load_x(x0, 0);
-        for (int blk = b0; blk < b1; ++blk) {
+        // The input rows are waited for here, once (with the first block's weights, requested before them and needed next
+        // anyway).  Left to the compiler, the wait sits in front of every multiply of every block - it cannot tell the
+        // first trip of the loop from the others - and, the rows being the newest loads it knows of, that wait covers the
+        // next block's weights as well: no block's loads would overlap the multiply of the block before.
+#pragma unroll
+        for (int s = 0; s < 16; ++s) asm volatile("" : "+v"(x0[s]));
+        // WITH_NEXT: the registers of a row take the next block's row as soon as the row is in LDS.  The last block is a
+        // copy of the code without those requests, not a condition around them (a load under a condition makes every
+        // wait of the loop assume the path without it and wait for more than it needs).
+        auto block = [&](int blk, auto with_next) {
             u32x4 op[16];
-            const bool more = blk + 1 < b1;
-            {
-                const half_t* next = a.W + (size_t)((more ? blk + 1 : blk) * 16) * a.K + k0 + lane * 8;
+            const half_t* next = a.W + (size_t)((blk + 1) * 16) * a.K + k0 + lane * 8;
 #pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    *reinterpret_cast<u32x4*>(mine + j * kMfmaFullRowBytes + lane * 16) = w[j];
-                    if (more) w[j] = ld_stream16(next + (size_t)j * a.K);
-                    asm volatile("" ::: "memory");        // keep the store / request pairs in this order
-                }
-                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-#pragma unroll
-                for (int s = 0; s < 16; ++s)
-                    op[s] = *reinterpret_cast<const u32x4*>(mine + (lane & 15) * kMfmaFullRowBytes + s * 64 + (lane >> 4) * 16);
-                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            for (int j = 0; j < 16; ++j) {
+                *reinterpret_cast<u32x4*>(mine + j * kMfmaFullRowBytes + lane * 16) = w[j];
+                if constexpr (decltype(with_next)::value) w[j] = ld_stream16(next + (size_t)j * a.K);
+                asm volatile("" ::: "memory");        // keep the store / request pairs in this order
             }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                op[s] = *reinterpret_cast<const u32x4*>(mine + (lane & 15) * kMfmaFullRowBytes + s * 64 + (lane >> 4) * 16);
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
             multiply(op, x0, blk, 0);
-        }
+        };
+        for (int blk = b0; blk + 1 < b1; ++blk) block(blk, std::true_type{});
+        block(b1 - 1, std::false_type{});
     } else {
         u32x4 wa[16], wb[16];
         request(wa, b0);
@@ -1210,45 +1218,77 @@ struct BatchAttn {
     const float* cos_sin;                                  // [positions][D]: cos of the D/2 pair angles, then sin
 };
 // One wave per (sequence, head, split); the parameter block of the single-sequence kernels, re-pointed at the
-// sequence's rows.
+// sequence's rows.  With one, two or four split slots per head the four waves of a workgroup hold whole heads, and a
+// head's partial results meet in LDS behind a workgroup barrier instead of in scratch memory behind a counter (three
+// dependent memory round trips less at the end of every item).
 __global__ __launch_bounds__(kStreamers * 64) void k_batch_attn(LayerParams p, BatchAttn b) {
+    touch_kernel_arguments<kLayerKernargBytes>();
+    __shared__ AttnLdsPart parts[kStreamers];
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
     const int item = blockIdx.x * kStreamers + wave;
     const int slots = p.max_split;                          // item slots per head (split 0 carries the new token)
+    const bool in_wg = slots == 1 || slots == 2 || slots == 4;
     const int per_seq = p.heads * slots;
     const int seq = item / per_seq;
-    if (seq >= b.batch) return;
+    bool active = seq < b.batch;
     const int rem = item - seq * per_seq;
     const int head = rem / slots, sp = rem - head * slots;
-    const int start = b.indptr[seq];
-    int S = b.indptr[seq + 1] - 1 - start;
-    if (S < 0) {
-        if (lane == 0) raise_status(status_sink(p), kStatusSeq);
-        return;
+    int S = 0, nsplit = 1, start = 0;
+    if (active) {
+        start = b.indptr[seq];
+        S = b.indptr[seq + 1] - 1 - start;
+        if (S < 0) {
+            if (lane == 0) raise_status(status_sink(p), kStatusSeq);
+            active = false;
+        } else {
+            nsplit = effective_split(p, S);
+            active = sp < nsplit;
+        }
     }
-    const int nsplit = effective_split(p, S);
-    if (sp >= nsplit) return;
+    if (!in_wg && !active) return;
     LayerParams q = p;
-    q.kv_rows = b.indices + start;
-    // The cache addresses come out of a table, so the compiler cannot see what kind of memory they point to and would
-    // use generic-address loads, whose completion it cannot count: every wait would then be for all loads in flight.
-    // Naming the address space (device memory) keeps them ordinary global loads.
-    typedef __attribute__((address_space(1))) half_t* GlobalHalf;
-    q.k_cache = (half_t*)(GlobalHalf)b.k_ptrs[b.layer_id];
-    q.v_cache = (half_t*)(GlobalHalf)b.v_ptrs[b.layer_id];
-    q.cos = b.cos_sin + (size_t)b.positions[seq] * p.D;
-    q.sin = q.cos + p.D / 2;
-    q.rope_stride = 0;
-    q.qkv_raw += (size_t)seq * 3 * p.H;
-    q.attn_vec += (size_t)seq * p.H;
-    q.k_new += (size_t)seq * p.H;
-    q.v_new += (size_t)seq * p.H;
-    q.part_ml += (size_t)seq * p.heads * kMaxSplit * 2;
-    q.part_acc += (size_t)seq * p.heads * kMaxSplit * p.D;
-    q.head_cnt += (size_t)seq * p.heads * kHeadCntStride;
-    AttnItem it;
-    attn_prefetch<true>(q, it, head, sp, nsplit, SeqLen{S, true}, lane);
-    attention_item<true>(q, it, lane, 0, 0);
+    if (active) {
+        q.kv_rows = b.indices + start;
+        // The cache addresses come out of a table, so the compiler cannot see what kind of memory they point to and would
+        // use generic-address loads, whose completion it cannot count: every wait would then be for all loads in flight.
+        // Naming the address space (device memory) keeps them ordinary global loads.
+        typedef __attribute__((address_space(1))) half_t* GlobalHalf;
+        q.k_cache = (half_t*)(GlobalHalf)b.k_ptrs[b.layer_id];
+        q.v_cache = (half_t*)(GlobalHalf)b.v_ptrs[b.layer_id];
+        q.cos = b.cos_sin + (size_t)b.positions[seq] * p.D;
+        q.sin = q.cos + p.D / 2;
+        q.rope_stride = 0;
+        q.qkv_raw += (size_t)seq * 3 * p.H;
+        q.attn_vec += (size_t)seq * p.H;
+        q.k_new += (size_t)seq * p.H;
+        q.v_new += (size_t)seq * p.H;
+        q.part_ml += (size_t)seq * p.heads * kMaxSplit * 2;
+        q.part_acc += (size_t)seq * p.heads * kMaxSplit * p.D;
+        q.head_cnt += (size_t)seq * p.heads * kHeadCntStride;
+        AttnItem it;
+        attn_prefetch<true>(q, it, head, sp, nsplit, SeqLen{S, true}, lane);
+        attention_item<true>(q, it, lane, 0, 0, in_wg ? &parts[wave] : nullptr);
+    }
+    if (!in_wg) return;
+    __syncthreads();
+    if (active && sp == 0) {
+        // the head's splits are waves wave .. wave + nsplit - 1; lane l merges dims 2 l and 2 l + 1, in split order
+        float M = kNegBig;
+        for (int i = 0; i < nsplit; ++i) M = fmaxf(M, parts[wave + i].m);
+        const int t2 = lane * 2;
+        const bool dact = t2 < p.D;
+        float L = 0.f, A0 = 0.f, A1 = 0.f;
+        for (int i = 0; i < nsplit; ++i) {
+            const float sc = fast_exp2(parts[wave + i].m - M);
+            L += parts[wave + i].l * sc;
+            A0 = fmadd(parts[wave + i].acc[dact ? t2 : 0], sc, A0);
+            A1 = fmadd(parts[wave + i].acc[dact ? t2 + 1 : 0], sc, A1);
+        }
+        if (dact) {
+            const half2_t o = {(half_t)(A0 / L), (half_t)(A1 / L)};
+            *reinterpret_cast<half2_t*>(q.attn_vec + (size_t)head * p.D + t2) = o;
+        }
+    }
 }
 
 
