@@ -404,10 +404,11 @@ def bench_llama_batch(args, emit=True):
         "ms_per_step": round(us * 1e-3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": f"llama2_7b attention block, {B} sequences x {S} cached tokens over paged caches (page = 1 token, "
-                               "scattered), 4 launches per call", "batch": B, "context": S, "hidden": H,
+                               f"scattered), {3 if B <= 16 else 4} launches per call", "batch": B, "context": S, "hidden": H,
                    "tokens_per_s_per_layer": round(B / (us * 1e-6))},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": None, "kernel": "k_batch_norm + k_batch_mfma_pipe (QKV) + k_batch_attn + k_batch_mfma_pipe (O)",
+                     "traffic": None, "kernel": ("k_batch_mfma_pipe (add + norm + QKV) + k_batch_attn + k_batch_mfma_pipe (O)" if B <= 16 else
+                                                  "k_batch_norm + k_batch_mfma_pipe (QKV) + k_batch_attn + k_batch_mfma_pipe (O)"),
                      "bytes_per_launch": nbytes, "launch_us": round(us, 2)},
         "cpu_baseline": None}
     if emit:

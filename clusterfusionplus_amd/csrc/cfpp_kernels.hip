@@ -870,6 +870,12 @@ struct BatchMfma {
     const half_t* x;                   // [batch][K]
     float* out_f32; half_t* out_f16;   // [batch][R], one of the two
     int batch;
+    // k_batch_mfma_pipe with up to 16 sequences, norm_w not null: the rows of x are raw; the product is taken with
+    // fp16(r * norm_w), r = fp16(x + x_add), and scaled by rstd(r) afterwards (the RMSNorm of r, with its one factor per
+    // sequence applied to the sums instead of to every element); r goes to sum_out.  x_add and sum_out are not null then.
+    const half_t *x_add, *norm_w;
+    half_t* sum_out;
+    float eps;
 };
 template <int KSTEPS>
 __global__ __launch_bounds__(512) void k_batch_mfma(BatchMfma a) {
@@ -955,6 +961,7 @@ __global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
         }
     };
     // multiply with one group of 16 sequences, add the NW partial sums up, store
+    float rs = 1.f;        // factor on the sums of sequence lane % 16 (the RMSNorm's, when this launch takes the norm)
     auto multiply = [&](const u32x4 (&op)[16], const u32x4 (&x)[16], int blk, int t0) {
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -967,6 +974,7 @@ __global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
             float sum = 0.f;
 #pragma unroll
             for (int u = 0; u < NW; ++u) sum += red[u][lane][wave];
+            sum *= rs;
             const int seq = t0 + (lane & 15), row = blk * 16 + 4 * (lane >> 4) + wave;
             if (seq < a.batch) {
                 const size_t o = (size_t)seq * a.R + row;
@@ -982,7 +990,56 @@ __global__ __launch_bounds__(NW * 64) void k_batch_mfma_pipe(BatchMfma a) {
         // fifteen or sixteen instead of draining to none once per block
         u32x4 w[16], x0[16];
         request(w, b0);
-        load_x(x0, 0);
+        if (a.norm_w == nullptr) {
+            load_x(x0, 0);
+        } else {
+            // Every workgroup takes the add + RMSNorm of the rows upon itself while its first weights travel (no launch for
+            // the norm).  A wave loads its 512-column share of all sixteen rows row by row (1 KB per load instruction, as
+            // it loads the weights), leaves r * norm_w in its staging buffer and reads the operand layout back, the way
+            // the weight blocks go.  No wave waits for another before the products start: the factor rstd, one per
+            // sequence, which needs the whole row, is applied to the sums.  Workgroup 0 stores the rows r.
+            __shared__ float ssq[NW][16];
+            const size_t col = k0 + lane * 8;
+            const u32x4 gw = ld16(a.norm_w + col);
+            u32x4 xa[16], xb[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) xa[r] = ld16(a.x + (size_t)(r < a.batch ? r : a.batch - 1) * a.K + col);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) xb[r] = ld16(a.x_add + (size_t)(r < a.batch ? r : a.batch - 1) * a.K + col);
+            // fp16 pair arithmetic: the sum of two fp16 values and the product of two fp16 values are exact in fp32, so
+            // rounding them once to fp16 is what the pair instructions do as well; the squares are summed in fp32
+            float mine_ss = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t ax[4] = {xa[r].x, xa[r].y, xa[r].z, xa[r].w}, bx[4] = {xb[r].x, xb[r].y, xb[r].z, xb[r].w};
+                const uint32_t gx[4] = {gw.x, gw.y, gw.z, gw.w};
+                uint32_t rr[4], yy[4];
+                float ss = 0.f;
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const half2_t t = as_h2(ax[q4]) + as_h2(bx[q4]);
+                    rr[q4] = as_u32(t);
+                    ss = __builtin_amdgcn_fdot2(t, t, ss, false);
+                    yy[q4] = as_u32(t * as_h2(gx[q4]));
+                }
+                const u32x4 rv = {rr[0], rr[1], rr[2], rr[3]}, yv = {yy[0], yy[1], yy[2], yy[3]};
+                if (blockIdx.x == 0 && r < a.batch) *reinterpret_cast<u32x4*>(a.sum_out + (size_t)r * a.K + col) = rv;
+                ss = wave_sum(ss);
+                if (lane == r) mine_ss = ss;
+                *reinterpret_cast<u32x4*>(mine + r * kMfmaFullRowBytes + lane * 16) = yv;
+            }
+            if (lane < 16) ssq[wave][lane] = mine_ss;
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                x0[s] = *reinterpret_cast<const u32x4*>(mine + (lane & 15) * kMfmaFullRowBytes + s * 64 + (lane >> 4) * 16);
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __syncthreads();
+            float tot = 0.f;
+#pragma unroll
+            for (int u = 0; u < NW; ++u) tot += ssq[u][lane & 15];
+            rs = 1.0f / sqrtf(tot / (float)a.K + a.eps);
+        }
         // The input rows are waited for here, once (with the first block's weights, requested before them and needed next
         // anyway).  Left to the compiler, the wait sits in front of every multiply of every block - it cannot tell the
         // first trip of the loop from the others - and, the rows being the newest loads it knows of, that wait covers the
@@ -1801,6 +1858,8 @@ int launch_batch_mfma(const BatchMfma& a, hipStream_t st) {
     hipLaunchKernelGGL((k_batch_mfma<4>), dim3(grid), dim3(512), 0, st, a);
     return (int)hipGetLastError();
 }
+// the kernel that takes the norm of the rows upon itself: the pipelined one, with its input rows kept in registers
+bool batch_mfma_norm_inside(int k, int batch) { return (k == 4096 || k == 2048) && batch <= 16; }
 bool batch_mfma_supported(int rows, int k) { return rows % 16 == 0 && k % 256 == 0 && (k == 1024 || k == 2048 || k == 4096); }
 int launch_batch_norm(int nch, const BatchNorm& a, hipStream_t st) {
     const dim3 grid((a.batch + kStreamers - 1) / kStreamers), block(kStreamers * 64);
@@ -2135,15 +2194,21 @@ int cfpp_llama_batch_decode(const cfpp_llama_batch* a, void* workspace, size_t w
     const bool mfma = batch_mfma_supported(d.hidden, d.hidden) && a->batch >= 2;
     CFPP_REFUSE_AFTER_FAILURE();
     if (mfma) {
-        BatchNorm n{};
-        n.x = h(a->input); n.x_add = h(a->residual); n.norm_w = h(a->rms_w);
-        n.sum_out = reinterpret_cast<half_t*>(a->residual_out); n.y = reinterpret_cast<half_t*>(ws + L.x_norm);
-        n.eps = a->eps; n.K = d.hidden; n.batch = a->batch;
-        if ((rc = launch_batch_norm(nch, n, st))) return rc;
         BatchMfma m{};
         m.W = h(a->w_qkv); m.R = 3 * d.hidden; m.K = d.hidden;
-        m.x = reinterpret_cast<const half_t*>(ws + L.x_norm);
         m.out_f32 = reinterpret_cast<float*>(ws + L.qkv_raw); m.out_f16 = nullptr; m.batch = a->batch;
+        if (batch_mfma_norm_inside(d.hidden, a->batch)) {
+            // up to 16 sequences: every workgroup of the QKV launch takes the norm upon itself (no launch for it)
+            m.x = h(a->input); m.x_add = h(a->residual); m.norm_w = h(a->rms_w);
+            m.sum_out = reinterpret_cast<half_t*>(a->residual_out); m.eps = a->eps;
+        } else {
+            BatchNorm n{};
+            n.x = h(a->input); n.x_add = h(a->residual); n.norm_w = h(a->rms_w);
+            n.sum_out = reinterpret_cast<half_t*>(a->residual_out); n.y = reinterpret_cast<half_t*>(ws + L.x_norm);
+            n.eps = a->eps; n.K = d.hidden; n.batch = a->batch;
+            if ((rc = launch_batch_norm(nch, n, st))) return rc;
+            m.x = reinterpret_cast<const half_t*>(ws + L.x_norm);
+        }
         if ((rc = launch_batch_mfma(m, st))) return rc;
     }
     BatchGemv g{};
