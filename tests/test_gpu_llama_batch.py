@@ -79,6 +79,15 @@ def test_small_geometry_repeatable_and_page_order(cf):
     assert torch.equal(r1[1], r2[1])
 
 
+@pytest.mark.parametrize("lens", [[200, 0, 33, 1, 90], [17] * 20, [300] * 16])
+def test_hidden_2048_geometry(cf, lens):
+    """hidden 2048, 16 heads of 128: the four-wave instantiation of the pipelined row kernel; up to 16 sequences with the
+    norm inside the QKV launch and the heads merged inside a workgroup, more than 16 with the norm as a launch of its own."""
+    print(f"\ncase llama paged batch hidden=2048 lens={lens}", flush=True)
+    dims = O.LlamaDims(hidden=2048, heads=16, head_dim=128, ffn=0)
+    check(*run(cf, dims, lens, seed=7 + len(lens), w_std=0.03))
+
+
 def test_batch_of_one_equals_single_sequence_op(cf):
     """With an identity page table the batched op and `llama_decoder_layer_sglang` see the same problem."""
     print("\ncase paged batch of one vs single-sequence op", flush=True)
