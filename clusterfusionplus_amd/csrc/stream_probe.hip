@@ -5,7 +5,9 @@
 //      unit (4 or 7; an eighth wave times a chain of dependent returning atomics / coherent loads, which is what every
 //      hop of a device-wide event or of the attention chain is) and by the load instructions each wave keeps in flight
 //      (1 KB each: 8 KB rows, non-temporal 16-byte lane loads, as the weight streams of the layer kernels);
-//   2. a region read again after a warm-up pass against the same region read cold (another gigabyte read in between):
+//   2. the same streams with the address of every piece worked out slightly differently (same rows, or rows interleaved
+//      with an odd stride, or a contiguous range per wave): how much of the rates of 1. is the exact instruction stream;
+//   3. a region read again after a warm-up pass against the same region read cold (another gigabyte read in between):
 //      what the 256 MB memory-side cache is worth to a weight stream.
 #include <hip/hip_runtime.h>
 
@@ -22,17 +24,25 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // D load instructions in flight per streaming wave, issued in two half batches; `nstream` streaming waves per
 // workgroup (one workgroup of eight waves per compute unit); wave 7 times `hops` dependent round trips.
-template <int D>
+// VARIANT: the same rows for the same waves (pad 0, contiguous 0), but the address of a piece is worked out with a
+// run-time choice of the row order in it: rows of the waves interleaved with a stride of waves + pad rows, or a
+// contiguous range per wave.
+template <int D, bool VARIANT = false>
 __global__ __launch_bounds__(512) void k_stream(const u32x4* __restrict__ w, int nrows, int nstream, int* ctr, int hops, float* lat,
-                                                unsigned* out, int coherent_load) {
+                                                unsigned* out, int coherent_load, int pad = 0, int contiguous = 0) {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     constexpr int HB = D / 2;
     if (wave < nstream) {
         const int gw = blockIdx.x * nstream + wave, nw = gridDim.x * nstream;
         unsigned acc = 0;
         // piece i of this wave: 1 KB, eight consecutive pieces are one 8 KB row; the rows of the waves interleave
-        auto addr = [&](size_t i) { const size_t row = (i / 8) * nw + gw; return w + (row * 8 + i % 8) * 64 + lane; };
-        const size_t mine = (size_t)(nrows / nw) * 8;
+        const size_t per = (size_t)(nrows / (nw + pad));
+        auto addr = [&](size_t i) {
+            size_t row = (i / 8) * nw + gw;
+            if (VARIANT) row = contiguous ? (size_t)gw * per + i / 8 : (i / 8) * (size_t)(nw + pad) + gw;
+            return w + (row * 8 + i % 8) * 64 + lane;
+        };
+        const size_t mine = per * 8;
         u32x4 a[HB], b[HB];
 #pragma unroll
         for (int u = 0; u < HB; ++u) a[u] = __builtin_nontemporal_load(addr(u));
@@ -99,14 +109,15 @@ __global__ __launch_bounds__(512) void k_rows(const u32x4* __restrict__ p, int n
     if (acc == 0x12345678u) out[0] = acc;
 }
 
-template <int D>
+template <int D, bool VARIANT = false>
 int run_stream(const std::vector<u32x4*>& bufs, int& turn, int nrows, int grid, int nstream, int hops, int coherent, int* ctr, float* lat,
-               unsigned* out, hipEvent_t e0, hipEvent_t e1) {
+               unsigned* out, hipEvent_t e0, hipEvent_t e1, int pad = 0, int contiguous = 0) {
     CHECK(hipMemset(lat, 0, grid * sizeof(float)));
     float best = 1e9f;
     for (int it = 0; it < 6; ++it) {
         CHECK(hipEventRecord(e0));
-        hipLaunchKernelGGL((k_stream<D>), dim3(grid), dim3(512), 0, 0, bufs[(turn++) % bufs.size()], nrows, nstream, ctr, hops, lat, out, coherent);
+        hipLaunchKernelGGL((k_stream<D, VARIANT>), dim3(grid), dim3(512), 0, 0, bufs[(turn++) % bufs.size()], nrows, nstream, ctr, hops, lat, out, coherent,
+                           pad, contiguous);
         CHECK(hipEventRecord(e1));
         CHECK(hipEventSynchronize(e1));
         float ms = 0.f;
@@ -117,7 +128,8 @@ int run_stream(const std::vector<u32x4*>& bufs, int& turn, int nrows, int grid, 
     CHECK(hipMemcpy(hl.data(), lat, grid * sizeof(float), hipMemcpyDeviceToHost));
     double s = 0, mx = 0;
     for (float x : hl) { s += x; if (x > mx) mx = x; }
-    const double bytes = (double)(grid * nstream) * (double)((nrows / (grid * nstream)) * 8) * 1024.0;
+    const double bytes = (double)(grid * nstream) * (double)((nrows / (grid * nstream + pad)) * 8) * 1024.0;
+    if (VARIANT) printf("[%s] ", contiguous ? "contiguous rows per wave" : pad ? "interleaved, stride waves + 1" : "interleaved, stride waves   ");
     printf("%2d loads (KB) in flight per wave, %d streaming waves per compute unit = %3d KB per compute unit: %6.1f us %.2f TB/s", D, nstream,
            D * nstream, best * 1e3, bytes / best / 1e9);
     if (hops > 0) printf(" ; dependent %s: mean %.2f us, slowest compute unit %.2f us", coherent ? "coherent load" : "returning atomic", s / grid, mx);
@@ -153,6 +165,15 @@ int main() {
         if (run_stream<16>(bufs, turn, nrows, grid, ns, 0, 0, ctr, lat, out, e0, e1)) return 1;
         if (run_stream<8>(bufs, turn, nrows, grid, ns, 0, 0, ctr, lat, out, e0, e1)) return 1;
     }
+    printf("\n[4] section [2] with the address arithmetic of the variant kernel (the first line of each group reads exactly the rows of\n"
+           "    section [2], wave by wave)\n");
+    for (int ns : {4, 7, 8})
+        for (int mode = 0; mode < 3; ++mode) {
+            const int pad = mode == 1, cont = mode == 2;
+            if (run_stream<32, true>(bufs, turn, nrows, grid, ns, 0, 0, ctr, lat, out, e0, e1, pad, cont)) return 1;
+            if (run_stream<16, true>(bufs, turn, nrows, grid, ns, 0, 0, ctr, lat, out, e0, e1, pad, cont)) return 1;
+            if (run_stream<8, true>(bufs, turn, nrows, grid, ns, 0, 0, ctr, lat, out, e0, e1, pad, cont)) return 1;
+        }
     printf("\n[3] a region read again after a warm-up pass, and read cold (1 GB of another buffer read in between); 8 waves per compute unit,\n"
            "    two 8 KB rows in flight per wave\n");
     u32x4 *big, *other;
