@@ -1167,6 +1167,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
             for (int j = 0; j < 8; ++j) q[j] *= p.qscale;
         }
 
+        trace_value(p, 8, wall_clock64() + (long long)(__builtin_bit_cast(unsigned, q[0]) & 0u));      // q is back and rotated
         auto process = [&](const KvTile& kv, int i) {
             const int r = it.begin + i * kAttnTileRows + grp;
             float s[kAttnT], mt = m;
@@ -1265,6 +1266,7 @@ __device__ __forceinline__ void attention_item(const LayerParams& p, AttnItem& i
     const int nparts = OWN_ITEM ? nsplit + 1 : nsplit;      // the cache items and the new token's item
     if (lane == 0) last = (__hip_atomic_fetch_add(p.head_cnt + head * kHeadCntStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nparts - 1);
     last = first_lane(last);
+    trace_mark(p, 11);       // partial published, head counter answered
     if (last) {
         // The last wave of this head merges the partial results.  Lane i fetches (m_i, l_i) of item i, so the
         // scales come from one round trip; the accumulators (two dims per lane) are fetched kMergeBatch

@@ -36,7 +36,9 @@ def load_trace_library(path):
 SLOTS = [(0, "kernel entry", "all"), (14, "LayerNorm inputs and first weight tile requested", "all"), (15, "own chunk of the input row arrived", "all"),
          (1, "LayerNorm done", "all"), (2, "own QKV rows stored, QKV arrival counted", "streaming"),
          (2, "own QKV rows stored, QKV arrival counted", "attention"),
-         (3, "QKV event seen, attention item begins", "attention"), (4, "attention item done (head merged by its last split)", "attention"),
+         (3, "QKV event seen, attention item begins", "attention"), (8, "item's q back and rotated (cache items)", "attention"),
+         (11, "item's partial published, head counter answered", "attention"),
+         (4, "attention item done (head merged by its last split)", "attention"),
          (12, "own MLP-up phase 0 rows stored", "streaming"), (5, "own MLP-up phase 1 rows stored", "streaming"),
          (6, "MLP-up phase 0 event seen (down phase 0 may read)", "streaming"), (13, "MLP-up phase 1 event seen (down phase 1 may read)", "streaming"),
          (7, "heads event seen (O rows may read)", "attention"), (9, "stage C begins", "all"), (10, "stage C done: rows reduced and stored", "all")]
@@ -139,7 +141,7 @@ def report(launches):
         us = (raw - t0) / 100.0
         for slot, label, who in SLOTS:
             sl = {"all": slice(0, 8), "streaming": slice(0, 4), "attention": slice(4, 8)}[who]
-            col = us[:, sl, slot][raw[:, sl, slot] > 0]
+            col = us[:, sl, slot][raw[:, sl, slot] >= t0]        # waves that do not pass a boundary leave its slot at zero
             if col.size:
                 rows.setdefault((slot, who), []).append((col.mean(), col.min(), np.percentile(col, 50), col.max()))
     print(f"{'phase boundary (us from the first wave; median over layers of ...)':84s} {'mean':>7s} {'first':>7s} {'median':>7s} {'last':>7s}")
