@@ -62,7 +62,8 @@ def check(ref, out, res_out, gc, caches, indptr, indices, layer_id):
         assert_close("new v rows", vc[slots], ref["v_cache"][slots])
 
 
-@pytest.mark.parametrize("lens", [[1024], [700, 3, 0, 129], [64] * 8, [2048, 1, 333, 17, 900, 5, 64, 1500, 31], [40] * 19])
+@pytest.mark.parametrize("lens", [[1024], [700, 3, 0, 129], [64] * 8, [2048, 1, 333, 17, 900, 5, 64, 1500, 31], [40] * 19,
+                                  [0, 5, 1024, 33] * 4, [1, 0] * 16])
 def test_llama2_7b_batch_matches_oracle(cf, lens):
     print(f"\ncase llama2-7b paged batch lens={lens}", flush=True)
     r = run(cf, O.LLAMA2_7B, lens, seed=len(lens), max_pos=4096)
