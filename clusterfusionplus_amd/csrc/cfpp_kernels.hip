@@ -585,7 +585,7 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
 }
 
 // ---- whole-model helpers -----------------------------------------------------------------------
-// hidden <- embed[token]
+// hidden <- embed[token]   (after the host has set the token; between steps the LM head's last workgroup does this)
 __global__ void k_embed(const half_t* __restrict__ embed, const int* __restrict__ state, int H, int vocab,
                         half_t* __restrict__ hidden) {
     int tok = state[0];
@@ -594,12 +594,25 @@ __global__ void k_embed(const half_t* __restrict__ embed, const int* __restrict_
     if (i < H) *reinterpret_cast<u32x4*>(hidden + i) = ld16(embed + (size_t)tok * H + i);
 }
 
-// logits = W LN(x); every workgroup also records its best (value, index) for the greedy pick
+// What the last workgroup of the LM head to finish does for a whole-model step: the greedy pick over the workgroups'
+// best (value, index) pairs, the step's bookkeeping, and the next token's embedding row.
+struct LmTail {
+    float* best_val;      // one pair per workgroup; nullptr: logits only
+    int* best_idx;
+    int* state;           // {token, seq_len, step, steps since creation}
+    int* done;            // workgroups that have recorded their pair; the last one sets it back to 0
+    int* history;
+    int hist_cap;
+    const half_t* embed;  // [vocab, H]
+    half_t* next_x;       // <- embed[token picked]
+};
+
+// logits = W LN(x); with a tail, token <- argmax, seq_len <- seq_len + 1, history[step] <- token, next_x <- embed[token]
 template <int NCH, bool EX>
 __global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __restrict__ x, int H, float eps,
                                                       const half_t* __restrict__ ln_w, const half_t* __restrict__ ln_b,
                                                       const half_t* __restrict__ W, int vocab, float* __restrict__ logits,
-                                                      float* __restrict__ best_val, int* __restrict__ best_idx) {
+                                                      LmTail tail) {
     touch_kernel_arguments<128>();
     constexpr int NWV = kStreamers;
     __shared__ float sv[NWV];
@@ -640,47 +653,53 @@ __global__ __launch_bounds__(kStreamers * 64) void k_lm_head(const half_t* __res
         const int oi = __shfl_xor(bi, m, kWave);
         if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
     }
+    if (tail.best_val == nullptr) return;
     if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
     __syncthreads();
+    __shared__ int last;
     if (threadIdx.x == 0) {
         for (int w = 1; w < NWV; ++w)
             if (sv[w] > bv || (sv[w] == bv && si[w] < bi)) { bv = sv[w]; bi = si[w]; }
-        if (best_val) { best_val[blockIdx.x] = bv; best_idx[blockIdx.x] = bi; }
+        st_agent(tail.best_val + blockIdx.x, bv);
+        st_agent(reinterpret_cast<uint32_t*>(tail.best_idx) + blockIdx.x, (uint32_t)bi);
+        drain_memory_ops();     // the pair is in memory before this workgroup counts as done
+        last = __hip_atomic_fetch_add(tail.done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (int)gridDim.x - 1;
     }
-}
-
-// token <- argmax, seq_len <- seq_len + 1, history[step] <- token   (one workgroup of 256 threads)
-__global__ __launch_bounds__(256) void k_pick_and_advance(const float* __restrict__ best_val, const int* __restrict__ best_idx,
-                                                          int n, int* __restrict__ state, int* __restrict__ history, int hist_cap) {
-    __shared__ float sv[4];
-    __shared__ int si[4];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    float bv = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) {
-        const float v = best_val[i];
-        const int r = best_idx[i];
+    __syncthreads();
+    if (!last) return;
+    // every workgroup has recorded its pair: pick over them (ties go to the lower index, whatever the reduction order)
+    bv = -INFINITY;
+    bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < (int)gridDim.x; i += NWV * 64) {
+        const float v = ld_agent(tail.best_val + i);
+        const int r = counter_peek(tail.best_idx + i);
         if (v > bv || (v == bv && r < bi)) { bv = v; bi = r; }
     }
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {     // ties go to the lower index, whatever the reduction order
-        const float ov = __shfl_xor(bv, m, kWave);
+    for (int m = 32; m >= 1; m >>= 1) {
+        const float ov = xor_shfl(bv, m);
         const int oi = __shfl_xor(bi, m, kWave);
         if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
     }
     if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
     __syncthreads();
+    for (int w = 0; w < NWV; ++w)
+        if (sv[w] > bv || (sv[w] == bv && si[w] < bi)) { bv = sv[w]; bi = si[w]; }
+    bi = bi < 0 ? 0 : (bi >= vocab ? vocab - 1 : bi);
+    for (int i = threadIdx.x * 8; i < H; i += NWV * 64 * 8)
+        *reinterpret_cast<u32x4*>(tail.next_x + i) = ld16(tail.embed + (size_t)bi * H + i);
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; ++w)
-            if (sv[w] > bv || (sv[w] == bv && si[w] < bi)) { bv = sv[w]; bi = si[w]; }
-        const int step = state[2];
-        state[0] = bi;
-        state[1] = state[1] + 1;
-        state[2] = step + 1;
-        state[3] = state[3] + 1;      // steps since the stack was created: never reset, launch tags derive from it
-        if (step < hist_cap) history[step] = bi;
+        const int step = tail.state[2];
+        tail.state[0] = bi;
+        tail.state[1] = tail.state[1] + 1;
+        tail.state[2] = step + 1;
+        tail.state[3] = tail.state[3] + 1;      // steps since the stack was created: never reset, launch tags derive from it
+        if (step < tail.hist_cap) tail.history[step] = bi;
+        __hip_atomic_store(tail.done, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
+
+constexpr int kStateDone = 8;   // word of the stack's state block that counts the LM head's finished workgroups
 
 __global__ void k_set_state(int* state, int token, int seq_len) {
     if (threadIdx.x == 0 && blockIdx.x == 0) { state[0] = token; state[1] = seq_len; state[2] = 0; }
@@ -2434,7 +2453,7 @@ int cfpp_ctx_destroy(int family, int64_t id) {
 // ---- LM head -------------------------------------------------------------------------------------
 namespace {
 int launch_lm_head(int H, int vocab, float eps, const void* x, const void* ln_w, const void* ln_b, const void* W,
-                   float* logits, float* best_val, int* best_idx, int grid, hipStream_t st) {
+                   float* logits, const LmTail& tail, int grid, hipStream_t st) {
     const int nch = (H + kChunk - 1) / kChunk;
     auto h = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
     switch (nch) {
@@ -2442,10 +2461,10 @@ int launch_lm_head(int H, int vocab, float eps, const void* x, const void* ln_w,
     case n:                                                                                                     \
         if (H == n * kChunk)                                                                                    \
             hipLaunchKernelGGL((k_lm_head<n, true>), dim3(grid), dim3(kStreamers * 64), 0, st, h(x), H, eps, h(ln_w),  \
-                               h(ln_b), h(W), vocab, logits, best_val, best_idx);                               \
+                               h(ln_b), h(W), vocab, logits, tail);                                             \
         else                                                                                                    \
             hipLaunchKernelGGL((k_lm_head<n, false>), dim3(grid), dim3(kStreamers * 64), 0, st, h(x), H, eps, h(ln_w), \
-                               h(ln_b), h(W), vocab, logits, best_val, best_idx);                               \
+                               h(ln_b), h(W), vocab, logits, tail);                                             \
         return launch_check();
         CFPP_NCH_CASES(X)
 #undef X
@@ -2463,7 +2482,7 @@ int cfpp_neox_lm_head(int32_t hidden, int32_t vocab, float eps, const void* x, c
     if (hidden <= 0 || hidden % 8 || hidden > 8 * kChunk || vocab <= 0 || vocab > kMaxVocab) return CFPP_ERR_DIMS;
     if (!aligned16(x) || !aligned16(ln_w) || !aligned16(ln_b) || !aligned16(w)) return CFPP_ERR_ALIGN;
     Plan pl{};
-    return launch_lm_head(hidden, vocab, eps, x, ln_w, ln_b, w, logits, nullptr, nullptr, grid_for_streaming(pl),
+    return launch_lm_head(hidden, vocab, eps, x, ln_w, ln_b, w, logits, LmTail{}, grid_for_streaming(pl),
                           reinterpret_cast<hipStream_t>(stream));
 }
 
@@ -2475,8 +2494,9 @@ struct cfpp_neox_stack {
     Plan plan{};
     int device = 0, grid = 0;
     char* slab = nullptr;
-    int* state = nullptr;         // {token, seq_len, step, steps since creation}
+    int* state = nullptr;         // {token, seq_len, step, steps since creation, ..., [kStateDone] LM-head workgroups done}
     half_t* hidden[2] = {nullptr, nullptr};
+    half_t* x0 = nullptr;         // embedding row of the current token: written by set_state, then by each step's LM head
     half_t *k_new = nullptr, *v_new = nullptr;
     float* logits = nullptr;
     float* best_val = nullptr;
@@ -2498,7 +2518,7 @@ namespace {
 cfpp_neox_io stack_layer_io(const cfpp_neox_stack* s, int l) {
     const cfpp_neox_dims& d = s->desc.dims;
     cfpp_neox_io io{};
-    io.input = s->hidden[l & 1];
+    io.input = l == 0 ? s->x0 : s->hidden[l & 1];
     io.output = s->hidden[(l + 1) & 1];
     io.k_new = s->k_new; io.v_new = s->v_new;
     io.k_cache = s->kc[l]; io.v_cache = s->vc[l];
@@ -2521,23 +2541,20 @@ int stack_enqueue_layer(cfpp_neox_stack* s, int l, hipStream_t st) {
     return run_layer(pl, p, s->desc.mode, seq_hint_of(&io), st);
 }
 
+LmTail stack_tail(const cfpp_neox_stack* s) {
+    return LmTail{s->best_val, s->best_idx, s->state, s->state + kStateDone, s->history, s->hist_cap,
+                  reinterpret_cast<const half_t*>(s->desc.embed), s->x0};
+}
+// one launch per layer and one for the LM head, whose last workgroup picks the token, advances the state and
+// fetches the picked token's embedding row for the next step
 int stack_enqueue_step(cfpp_neox_stack* s, hipStream_t st) {
     const cfpp_neox_dims& d = s->desc.dims;
-    const int H = d.hidden;
-    hipLaunchKernelGGL(k_embed, dim3((H / 8 + 255) / 256), dim3(256), 0, st,
-                       reinterpret_cast<const half_t*>(s->desc.embed), s->state, H, s->desc.vocab, s->hidden[0]);
-    int rc = launch_check();
-    if (rc) return rc;
     for (int l = 0; l < s->desc.n_layers; ++l) {
-        rc = stack_enqueue_layer(s, l, st);
+        const int rc = stack_enqueue_layer(s, l, st);
         if (rc) return rc;
     }
-    rc = launch_lm_head(H, s->desc.vocab, d.eps, s->hidden[s->desc.n_layers & 1], s->desc.final_ln_w, s->desc.final_ln_b,
-                        s->desc.lm_head, s->logits, s->best_val, s->best_idx, s->grid, st);
-    if (rc) return rc;
-    hipLaunchKernelGGL(k_pick_and_advance, dim3(1), dim3(256), 0, st, s->best_val, s->best_idx, s->grid, s->state,
-                       s->history, s->hist_cap);
-    return launch_check();
+    return launch_lm_head(d.hidden, s->desc.vocab, d.eps, s->hidden[s->desc.n_layers & 1], s->desc.final_ln_w,
+                          s->desc.final_ln_b, s->desc.lm_head, s->logits, stack_tail(s), s->grid, st);
 }
 }  // namespace
 
@@ -2565,6 +2582,7 @@ int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out) {
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
     const size_t o_state = take(64), o_h0 = take((size_t)d.hidden * 2), o_h1 = take((size_t)d.hidden * 2);
+    const size_t o_x0 = take((size_t)d.hidden * 2);
     const size_t o_k = take((size_t)d.hidden * 2), o_v = take((size_t)d.hidden * 2);
     const size_t o_logits = take((size_t)desc->vocab * 4);
     const size_t o_bv = take((size_t)s->grid * 4), o_bi = take((size_t)s->grid * 4);
@@ -2578,6 +2596,7 @@ int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out) {
     s->state = reinterpret_cast<int*>(s->slab + o_state);
     s->hidden[0] = reinterpret_cast<half_t*>(s->slab + o_h0);
     s->hidden[1] = reinterpret_cast<half_t*>(s->slab + o_h1);
+    s->x0 = reinterpret_cast<half_t*>(s->slab + o_x0);
     s->k_new = reinterpret_cast<half_t*>(s->slab + o_k);
     s->v_new = reinterpret_cast<half_t*>(s->slab + o_v);
     s->logits = reinterpret_cast<float*>(s->slab + o_logits);
@@ -2585,6 +2604,12 @@ int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out) {
     s->best_idx = reinterpret_cast<int*>(s->slab + o_bi);
     s->history = reinterpret_cast<int*>(s->slab + o_hist);
     s->ws = s->slab + o_ws;
+    // the state block starts as token 0 at position 0: its embedding row, so that steps without set_state are defined
+    hipLaunchKernelGGL(k_embed, dim3((d.hidden / 8 + 255) / 256), dim3(256), 0, nullptr,
+                       reinterpret_cast<const half_t*>(desc->embed), s->state, d.hidden, desc->vocab, s->x0);
+    e = hipGetLastError();
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+    if (e != hipSuccess) { (void)hipFree(s->slab); delete s; return (int)e; }
     *out = s;
     return CFPP_OK;
 }
@@ -2593,8 +2618,14 @@ int cfpp_stack_set_state(cfpp_neox_stack* s, int32_t token, int32_t seq_len, voi
     if (!s) return CFPP_ERR_NULL;
     if (seq_len < 0 || seq_len >= s->desc.cache_rows) return CFPP_ERR_SEQ;     // the next step appends row seq_len
     if (token < 0 || token >= s->desc.vocab) return CFPP_ERR_DIMS;
-    hipLaunchKernelGGL(k_set_state, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(stream), s->state, token, seq_len);
-    const int rc = launch_check();
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(k_set_state, dim3(1), dim3(64), 0, st, s->state, token, seq_len);
+    int rc = launch_check();
+    if (rc) return rc;
+    const int H = s->desc.dims.hidden;
+    hipLaunchKernelGGL(k_embed, dim3((H / 8 + 255) / 256), dim3(256), 0, st,
+                       reinterpret_cast<const half_t*>(s->desc.embed), s->state, H, s->desc.vocab, s->x0);
+    rc = launch_check();
     if (!rc) s->host_seq_len = seq_len;
     return rc;
 }
@@ -2681,11 +2712,7 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
     int rc = CFPP_OK;
     {
         const cfpp_neox_dims& d = s->desc.dims;
-        const int H = d.hidden;
         CFPP_HIP(hipEventRecord(ev[L + 2], st));     // start of the step
-        hipLaunchKernelGGL(k_embed, dim3((H / 8 + 255) / 256), dim3(256), 0, st,
-                           reinterpret_cast<const half_t*>(s->desc.embed), s->state, H, s->desc.vocab, s->hidden[0]);
-        rc = launch_check();
         for (int l = 0; l < L && !rc; ++l) {
             CFPP_HIP(hipEventRecord(ev[l], st));
             if (fused) tl_kernel_events = &kev[l];
@@ -2694,11 +2721,9 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
         }
         if (!rc) {
             CFPP_HIP(hipEventRecord(ev[L], st));
-            rc = launch_lm_head(H, s->desc.vocab, d.eps, s->hidden[L & 1], s->desc.final_ln_w, s->desc.final_ln_b,
-                                s->desc.lm_head, s->logits, s->best_val, s->best_idx, s->grid, st);
+            rc = launch_lm_head(d.hidden, s->desc.vocab, d.eps, s->hidden[L & 1], s->desc.final_ln_w, s->desc.final_ln_b,
+                                s->desc.lm_head, s->logits, stack_tail(s), s->grid, st);
             CFPP_HIP(hipEventRecord(ev[L + 1], st));
-            hipLaunchKernelGGL(k_pick_and_advance, dim3(1), dim3(256), 0, st, s->best_val, s->best_idx, s->grid, s->state,
-                               s->history, s->hist_cap);
         }
     }
     hipEvent_t end;

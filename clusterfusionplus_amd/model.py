@@ -201,7 +201,8 @@ class NeoxDecoder:
 
     @property
     def state(self) -> torch.Tensor:
-        """int32 `[token, seq_len, steps_done]` on the device."""
+        """int32 `[token, seq_len, steps_done]` on the device; to read, not to write (`set_state` also fetches the
+        token's embedding row, which every step after it hands to the next one)."""
         return self._stack.state()
 
     def check(self):

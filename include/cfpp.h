@@ -320,11 +320,13 @@ typedef struct cfpp_neox_stack cfpp_neox_stack;   /* opaque */
 
 /* Allocates state (device int32 seq_len + token, hidden ping-pong, logits, workspace). */
 int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out);
-/* Sets the device-resident (token, seq_len) the next step starts from (async on `stream`); seq_len < cache_rows.
- * The step calls below return CFPP_ERR_SEQ instead of running past the last cache row. */
+/* Sets the device-resident (token, seq_len) the next step starts from and fetches that token's embedding row
+ * (async on `stream`); seq_len < cache_rows.  The step calls below return CFPP_ERR_SEQ instead of running past
+ * the last cache row. */
 int cfpp_stack_set_state(cfpp_neox_stack* s, int32_t token, int32_t seq_len, void* stream);
 /* One decode step launched eagerly: consumes (token, seq_len), appends K/V rows, writes logits,
- * then stores argmax as the new token and seq_len+1. */
+ * then stores argmax as the new token and seq_len+1 and fetches the new token's embedding row (the LM head
+ * launch does all of that: a step is n_layers + 1 launches in fused mode). */
 int cfpp_stack_step(cfpp_neox_stack* s, void* stream);
 /* Captures one step into a hipGraph (first call) and replays it `n_steps` times on `stream`. */
 int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream);
@@ -332,7 +334,8 @@ int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream);
  * `stream`; synchronises.  layer_ms[n_layers], *lm_head_ms and *total_ms (whole step) receive elapsed
  * milliseconds.  For measurement; advances the state like cfpp_stack_step. */
 int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, float* lm_head_ms, float* total_ms);
-/* Device pointers for inspection: logits fp32 [vocab], hidden fp16 [H] after the last layer,
+/* Device pointers for inspection (read only: the token is changed through cfpp_stack_set_state, which also
+ * fetches its embedding row): logits fp32 [vocab], hidden fp16 [H] after the last layer,
  * state int32[3] = {token, seq_len, steps done}, token history int32 [history_capacity]. */
 int cfpp_stack_buffers(cfpp_neox_stack* s, float** logits, void** hidden, int32_t** state,
                        int32_t** history, int32_t* history_capacity);
