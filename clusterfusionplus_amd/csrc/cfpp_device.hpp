@@ -189,6 +189,10 @@ __device__ __forceinline__ u32x4 ld_agent16(const void* p) {
     u32x4 r = {(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
     return r;
 }
+__device__ __forceinline__ half_t ld_agent(const half_t* p) {
+    const unsigned short u = __hip_atomic_load(reinterpret_cast<const unsigned short*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __builtin_bit_cast(half_t, u);
+}
 // all memory operations this wave has issued are complete
 __device__ __forceinline__ void drain_memory_ops() { __builtin_amdgcn_s_waitcnt(0); }
 
@@ -300,8 +304,10 @@ __device__ __forceinline__ int* group_counter(int* grp, int event, int g) {
 // workgroup arrive (1 if lds_ctr is null).  The wave that completes a count zeroes it for the next launch;
 // the one that completes the event writes `tag` into mailbox slot `event` of all `nwg` workgroups and
 // returns true.
-__device__ __forceinline__ bool event_arrive(int* bar, int* grp, int* mbox, int event, int nwg, int* lds_ctr, int per_wg, int tag) {
-    const int lane = threadIdx.x & 63;
+// (`lane_in`: the caller's lane index, for callers that keep it opaque to the optimiser.)
+__device__ __forceinline__ bool event_arrive(int* bar, int* grp, int* mbox, int event, int nwg, int* lds_ctr, int per_wg, int tag,
+                                             int lane_in = -1) {
+    const int lane = lane_in >= 0 ? lane_in : (int)(threadIdx.x & 63);
     drain_memory_ops();
     int go = 1;
     if (lds_ctr != nullptr) {
@@ -334,8 +340,8 @@ __device__ __forceinline__ bool event_arrive(int* bar, int* grp, int* mbox, int 
 // One lane polls this workgroup's mailbox line, the wave leaves together.  Data published before the
 // arrivals must be read with ld_agent / ld_agent16.  A wait that expires raises a status flag and
 // falls through.
-__device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, const StatusSink& status) {
-    if ((threadIdx.x & 63) == 0) {
+__device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, const StatusSink& status, int lane_in = -1) {
+    if ((lane_in >= 0 ? lane_in : (int)(threadIdx.x & 63)) == 0) {
         const int* f = mbox + blockIdx.x * kMailboxInts + slot;
         int spins = 0;
         while (counter_peek(f) != tag) {
@@ -344,6 +350,34 @@ __device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, c
         }
     }
     __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// The hand-over between two layers of one launch: every workgroup has its own flag word (the words are the group
+// counters of kBarExit, which such a launch does not count in: kLayerFlagWgs workgroups at most) and stores its
+// layer's tag there once its output rows are in memory; a waiting wave reads all the words with one load per lane
+// until none is behind.  No counter has to be carried through the memory side's atomic units on the way from the last
+// row stored to the first row read: two round trips less than an event.
+constexpr int kLayerFlagWgs = kEventGroups * kMailboxInts;
+__device__ __forceinline__ void layer_done_post(int* grp, int wg, int tag, int lane) {
+    drain_memory_ops();
+    if (lane == 0) st_agent(reinterpret_cast<uint32_t*>(group_counter(grp, kBarExit, 0)) + wg, (uint32_t)tag);
+}
+__device__ __forceinline__ void layer_done_wait(int* grp, int nwg, int tag, const StatusSink& status, int lane) {
+    const int* flags = group_counter(grp, kBarExit, 0);
+    int spins = 0;
+    for (;;) {
+        const u32x4 f = ld_agent16(flags + lane * 4);
+        const int i = lane * 4;
+        const bool ok = (i >= nwg || (int)(f.x - (uint32_t)tag) >= 0) && (i + 1 >= nwg || (int)(f.y - (uint32_t)tag) >= 0) &&
+                        (i + 2 >= nwg || (int)(f.z - (uint32_t)tag) >= 0) && (i + 3 >= nwg || (int)(f.w - (uint32_t)tag) >= 0);
+        if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+        __builtin_amdgcn_s_sleep(2);
+        if (++spins > kSpinLimit) {
+            if (lane == 0) raise_status(status, kStatusSpin);
+            break;
+        }
+    }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
@@ -419,14 +453,17 @@ __device__ __forceinline__ NormSpec norm_spec(const LayerParams& p) {
     return NormSpec{p.x, p.x_add, p.ln_w, p.ln_b, p.ln2_w, p.ln2_b, p.H, p.norm_rms, p.eps};
 }
 
-template <int NCH, int NW, bool TWO>
+// COH: the input rows were written earlier in this same launch by other workgroups (a launch that runs several layers):
+// they are read past the caches, like everything else that crosses workgroups inside a launch.
+template <int NCH, int NW, bool TWO, bool COH = false>
 __device__ __forceinline__ void ln_coop_load(LnOwn<NCH, NW>& o, const NormSpec& ns, int wave, int lane) {
     const u32x4 z = {0u, 0u, 0u, 0u};
+    auto row16 = [](const half_t* q) { if constexpr (COH) return ld_agent16(q); else return ld16(q); };
 #pragma unroll
     for (int k = 0; k < LnOwn<NCH, NW>::OWN; ++k) {
         const int col = (wave + k * NW) * kChunk + lane * 8;
         const bool in = wave + k * NW < NCH && col < ns.H;
-        o.rx[k] = in ? ld16(ns.x + col) : z;
+        o.rx[k] = in ? row16(ns.x + col) : z;
         o.rw1[k] = in ? ld16(ns.w1 + col) : z;
         o.rb1[k] = (in && ns.b1) ? ld16(ns.b1 + col) : z;
         if (TWO) {
@@ -435,7 +472,7 @@ __device__ __forceinline__ void ln_coop_load(LnOwn<NCH, NW>& o, const NormSpec& 
         }
         // the second input row, if there is one, is only requested here (without one, the first is requested again and
         // dropped): adding it up right away would make the wave wait for both rows before anything else can be requested
-        o.ra[k] = in ? ld16((ns.x_add != nullptr ? ns.x_add : ns.x) + col) : z;
+        o.ra[k] = in ? row16((ns.x_add != nullptr ? ns.x_add : ns.x) + col) : z;
     }
 }
 // x <- fp16(x + x_add), as the reference's fused add + RMSNorm does (reference include/5090/llama/kernel_sglang.cuh:98-105).
@@ -1475,9 +1512,12 @@ __device__ __forceinline__ void down_phases(const StageC& c, int ks, int lane, i
 // in flight and before its activations are read (the fused kernel waits for the producing event there).
 // The partials are added in a fixed order with the biases and residual terms: deterministic, and
 // identical in both modes.  Every wave of the workgroup must call this (workgroup barriers inside).
-template <int NCH, int CPD, class DownReady, class OReady>
+// COH: the layer's input rows (the residual terms) were written earlier in this same launch, and its output rows are
+// read later in it, by other workgroups: both go past the caches.
+template <int NCH, int CPD, bool COH = false, class DownReady, class OReady>
 __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, StageCShared& sh, bool streamer, int ks,
-                                             int o_index, int n_o, int lane, DownReady&& down_ready, OReady&& o_ready) {
+                                             int o_index, int n_o, int lane, DownReady&& down_ready, OReady&& o_ready,
+                                             int thread_in = -1) {
     const int r0 = mul_div(wg, c.nrows, nwg), r1 = mul_div(wg + 1, c.nrows, nwg);
     bool first = true;
     for (int b0 = r0; b0 < r1; b0 += kRowBatch) {
@@ -1489,18 +1529,19 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
         // compiler waited for each of them in turn, three or four dependent memory round trips in front of the first
         // weight tile of the wave that finishes the rows - it saw every event of the pass several microseconds after the
         // other waves, and the whole workgroup ended that much later.
-        const int et = (int)threadIdx.x;
+        const int et = thread_in >= 0 ? thread_in : (int)threadIdx.x;
         const bool finisher = et < b1 - b0;
         half_t h_b1, h_b2, h_x0, h_x1, h_sa, h_sb;      // (only read by the lanes that loaded them)
         if (first_lane(et >> 6) == 0) {     // the wave that holds the finishing lanes (a scalar branch)
             const int r = finisher ? b0 + et : b0;
             const half_t* any = c.out + r;
+            auto term = [](const half_t* q) { if constexpr (COH) return ld_agent(q); else return *q; };
             h_b1 = *(c.bias1 ? c.bias1 + r : any);
             h_b2 = *(c.bias2 ? c.bias2 + r : any);
-            h_x0 = *(c.base0 ? c.base0 + r : any);
-            h_x1 = *(c.base1 ? c.base1 + r : any);
-            h_sa = *((c.sum_b != nullptr || c.add_sum) ? c.sum_a + r : any);
-            h_sb = *(c.sum_b ? c.sum_b + r : any);
+            h_x0 = term(c.base0 ? c.base0 + r : any);
+            h_x1 = term(c.base1 ? c.base1 + r : any);
+            h_sa = term((c.sum_b != nullptr || c.add_sum) ? c.sum_a + r : any);
+            h_sb = term(c.sum_b ? c.sum_b + r : any);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (streamer && c.K2 > 0) down_phases<CPD, 0>(c, ks, lane, b0, b1, sh, first, down_ready);
@@ -1571,7 +1612,8 @@ __device__ __forceinline__ void stage_c_rows(const StageC& c, int wg, int nwg, S
                 if (c.sum_out) c.sum_out[r] = (half_t)rs;
                 if (c.add_sum) v += rs;
             }
-            c.out[r] = (half_t)v;
+            if constexpr (COH) st_agent(c.out + r, (half_t)v);
+            else c.out[r] = (half_t)v;
         }
         __syncthreads();
     }

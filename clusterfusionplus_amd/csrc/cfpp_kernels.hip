@@ -360,19 +360,29 @@ struct FusedLds {
 
 // One layer; `gen_word` is the word the launch tag derives from (the generation of the workspace, or the caller's step
 // counter), requested at the start of the launch.
-template <int NCH, int CPD, bool EX, bool BYX>
-__device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, FusedLds<NCH>& lds) {
+// CHAIN: the launch runs the layers of a whole model one after the other (k_fused_stack), and this is one of them.  Its
+// input row is the previous layer's output row, written by all workgroups: `wait_prev` makes the workgroup wait until all
+// of them have said so (layer_done_wait for the previous layer's tag, tag - 1), with the first weight tiles already
+// requested; `announce` makes it say so itself once its output rows are stored.  Rows that cross layers go past the caches.
+template <int NCH, int CPD, bool EX, bool BYX, bool CHAIN = false>
+__device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, FusedLds<NCH>& lds, bool wait_prev = false,
+                                            bool announce = false) {
     FusedShared& q = lds.q;
     StageCShared& shc = lds.shc;
     LnShared<NCH>& lns = lds.lns;
     float (&park_mem)[kStreamers][kParkRows] = lds.park_mem;
     int (&park_rows)[kStreamers][kParkRows] = lds.park_rows;
-    const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);   // wave index in a scalar register
+    int thread = threadIdx.x, lane_id = threadIdx.x & 63;
+    // In a loop over layers the compiler would work out everything that depends on the lane alone once, in front of the
+    // loop, and keep it in registers across all layers (two dozen of them, in a function that has none to spare):
+    // the lane index is made opaque per layer, so that those values are worked out where they are used.
+    if constexpr (CHAIN) asm volatile("" : "+v"(lane_id), "+v"(thread));
+    const int lane = lane_id, wave = first_lane(thread >> 6);   // wave index in a scalar register
     const int G = gridDim.x, b = blockIdx.x;
     const int nsw = G * kStreamers;                 // streaming waves in the grid
     const StatusSink status = status_sink(p);
     const int seq_requested = seq_len_request(p);     // on its way before anything else
-    if (threadIdx.x <= kUpPhases) q.arrived[threadIdx.x] = 0;
+    if (thread <= kUpPhases) q.arrived[thread] = 0;
     __syncthreads();
     trace_mark(p, 0);
     trace_value(p, 8, __builtin_amdgcn_s_getreg((3 << 11) | 20));   // XCC_ID: which XCD this workgroup runs on
@@ -400,9 +410,20 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
     // then starts when the slowest wave's tile has arrived instead of when the input row has.
     auto norm_phase = [&](auto with_tile) {
         LnOwn<NCH, kFusedWaves> own;
-        ln_coop_load<NCH, kFusedWaves, true>(own, norm_spec(p), wave, lane);
-        __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
-        if constexpr (decltype(with_tile)::value) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
+        if constexpr (CHAIN) {
+            // the weight tile does not depend on the previous layer: requested first, it is on its way while the last
+            // workgroups finish that layer.  One wave polls, the others wait for it at the barrier.
+            if constexpr (decltype(with_tile)::value) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
+            if (wait_prev) {
+                if (wave == kFusedWaves - 1) layer_done_wait(p.grp, G, first_lane(gen_word) * p.tag_mul + p.tag_add, status, lane);
+                __syncthreads();
+            }
+            ln_coop_load<NCH, kFusedWaves, true, true>(own, norm_spec(p), wave, lane);
+        } else {
+            ln_coop_load<NCH, kFusedWaves, true>(own, norm_spec(p), wave, lane);
+            __builtin_amdgcn_sched_barrier(0);   // the LayerNorm inputs go out first
+            if constexpr (decltype(with_tile)::value) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
+        }
         trace_mark(p, 14);
 #ifdef CFPP_TRACE
         trace_value(p, 15, wall_clock64() + (long long)(own.rx[0].x & 0u));     // the wave's chunk of the input row has arrived
@@ -452,7 +473,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
             drain_memory_ops();
             if (lane == 0) __hip_atomic_fetch_add(lds_ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         } else {
-            event_arrive(p.bar, p.grp, p.mbox, event, G, lds_ctr, kStreamers, tag);
+            event_arrive(p.bar, p.grp, p.mbox, event, G, lds_ctr, kStreamers, tag, lane);
         }
     };
     auto agent_serve = [&](int event, int* lds_ctr) {
@@ -464,7 +485,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
             }
         }
         __builtin_amdgcn_wave_barrier();
-        event_arrive(p.bar, p.grp, p.mbox, event, G, nullptr, 1, tag);
+        event_arrive(p.bar, p.grp, p.mbox, event, G, nullptr, 1, tag, lane);
     };
 
     if (wave < kStreamers) {
@@ -485,7 +506,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
         // at the hand-over is worth more than the earlier event (both orders measured, on both models).
         if (dynamic) {
             TeamTiles<NCH, kUpRpi> ut;
-            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
+            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag, lane);
             team_prefetch<NCH, kUpRpi, EX>(p.w_up, p.H, utm, lane, ut, p.b_up);
             trace_mark(p, 2);
             ln_fetch<NCH>(lns, 1, lane, xr);
@@ -502,7 +523,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
         } else {
             RowTile<NCH, kUpRpi> u0;
             RowWalk uw = row_walk<kUpRpi>(b * kStreamers + wave, nsw, 0, up_phase_rows(CPD, 0, p.F));
-            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
+            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag, lane);
             up_prefetch<NCH, EX>(p, uw, lane, u0);
             trace_mark(p, 2);
             ln_fetch<NCH>(lns, 1, lane, xr);
@@ -531,7 +552,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
             __builtin_amdgcn_s_setprio(2);
             qkv_rows<NCH, EX>(p, xq, qw, lane, t0, hpark);
             resolve();
-            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag);
+            event_arrive(p.bar, p.grp, p.mbox, kBarQkv, G, &q.arrived[0], qkv_arrivals, tag, lane);
             __builtin_amdgcn_s_setprio(0);
             trace_mark(p, 2);
         } else {
@@ -541,7 +562,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
             AttnItem it;
             const int item = item_lo + hw * item_step;
             attn_prefetch(p, it, head_lo + item / per_head, item % per_head, nsplit, sl, lane);
-            event_wait(p.mbox, kBarQkv, tag, status);
+            event_wait(p.mbox, kBarQkv, tag, status, lane);
             __builtin_amdgcn_s_setprio(3);   // few instructions, long dependent latencies: let them issue at once
             trace_mark(p, 3);
             attention_item(p, it, lane, G, tag);
@@ -558,15 +579,18 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
         const bool streamer = wave < kStreamers;
         // without an MLP-down pass (attention-only layers) all eight waves share the O-projection rows
         const bool all_o = c.K2 == 0;
-        stage_c_rows<NCH, CPD>(
+        stage_c_rows<NCH, CPD, CHAIN>(
             c, b, G, shc, streamer, wave, all_o ? wave : (streamer ? -1 : wave - kStreamers), all_o ? 2 * kStreamers : kStreamers, lane,
-            [&](int g) { event_wait(p.mbox, kBarUp + g, tag, status); trace_mark(p, g == 0 ? 6 : 13); },
-            [&] { event_wait(p.mbox, kBarHeads, tag, status); trace_mark(p, 7); });
+            [&](int g) { event_wait(p.mbox, kBarUp + g, tag, status, lane); trace_mark(p, g == 0 ? 6 : 13); },
+            [&] { event_wait(p.mbox, kBarHeads, tag, status, lane); trace_mark(p, 7); }, thread);
     }
     trace_mark(p, 10);
-    // the last workgroup to leave publishes the new generation: the flags of this launch turn stale
-    if (wave == 0 && p.tag_src == nullptr) {
-        const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1, tag);
+    if constexpr (CHAIN) {
+        // the wave that stored this workgroup's output rows raises the workgroup's flag for the next layer
+        if (wave == 0 && announce) layer_done_post(p.grp, b, tag, lane);
+    } else if (wave == 0 && p.tag_src == nullptr) {
+        // the last workgroup to leave publishes the new generation: the flags of this launch turn stale
+        const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1, tag, lane);
         if (last && lane == 0) __hip_atomic_store(p.bar + kBarGen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
@@ -582,6 +606,21 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     // (a vector load; nothing looks at the value until the wave has used up its first weight tile)
     const int gen_word = counter_peek(p.tag_src != nullptr ? p.tag_src : p.bar + kBarGen);
     fused_layer<NCH, CPD, EX, BYX>(p, gen_word, lds);
+}
+
+// All layers of a model in one launch: `table[l]` holds layer l's parameters (tags from the caller's step counter: tag_src
+// set, tag_add = l, so that consecutive layers have consecutive tags).  A workgroup that has finished a layer goes on to
+// the next one's first weight tiles while others are still busy, and the layers hand their rows over through an event
+// instead of a launch boundary.  All workgroups must be co-resident, as for k_fused.
+typedef __attribute__((address_space(4))) const LayerParams ConstLayerParams;
+template <int NCH, int CPD, bool EX, bool BYX>
+__global__ __launch_bounds__(2 * kStreamers * 64) void k_fused_stack(const LayerParams* table, int n_layers) {
+    __shared__ FusedLds<NCH> lds;
+    const int gen_word = first_lane(counter_peek(((ConstLayerParams*)table)->tag_src));     // the same word for every layer
+    for (int l = 0; l < n_layers; ++l) {
+        const LayerParams& p = *(const LayerParams*)((ConstLayerParams*)table + l);
+        fused_layer<NCH, CPD, EX, BYX, true>(p, gen_word, lds, l > 0, l + 1 < n_layers);
+    }
 }
 
 // ---- whole-model helpers -----------------------------------------------------------------------
@@ -1603,6 +1642,33 @@ int launch_fused_t(const LayerParams& p, int grid, hipStream_t st) {
 }
 template <int NCH, int CPD>
 bool fused_fits_t(const LayerParams& p, int grid) { return one_launch_fits(fused_fn<NCH, CPD>(p, grid), 2 * kStreamers * 64, grid); }
+// the same choice for the launch that runs all layers of a model
+template <int NCH, int CPD>
+const void* fused_stack_fn(const LayerParams& p, int grid) {
+    const bool byx = (p.D * 2) % 128 != 0 && p.heads % kXcds == 0 && grid % kXcds == 0;
+    // only for hidden sizes that fill their last 512-column chunk (the other instantiations do not fit the register file
+    // without spilling; such models take one launch per layer)
+    if (p.H != NCH * kChunk) return nullptr;
+    return byx ? (const void*)(k_fused_stack<NCH, CPD, true, true>) : (const void*)(k_fused_stack<NCH, CPD, true, false>);
+}
+template <int NCH, int CPD>
+int launch_fused_stack_t(const LayerParams& p0, const LayerParams* table, int n_layers, int grid, hipStream_t st) {
+    const void* fn = fused_stack_fn<NCH, CPD>(p0, grid);
+    if (fn == nullptr) return CFPP_ERR_DIMS;
+    void* args[] = {&table, &n_layers};
+    if (tl_kernel_events) {
+        CFPP_HIP(hipExtLaunchKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st, tl_kernel_events->start,
+                                    tl_kernel_events->stop, 0));
+        return CFPP_OK;
+    }
+    CFPP_HIP(hipLaunchKernel(fn, dim3(grid), dim3(2 * kStreamers * 64), args, 0, st));
+    return CFPP_OK;
+}
+template <int NCH, int CPD>
+bool fused_stack_fits_t(const LayerParams& p, int grid) {
+    const void* fn = fused_stack_fn<NCH, CPD>(p, grid);
+    return fn != nullptr && one_launch_fits(fn, 2 * kStreamers * 64, grid);
+}
 
 // hidden chunks that occur in CFPP_SHAPE_CASES below (both lists can be narrowed on the compiler's command line for a
 // quick experimental build; the shapes left out are then refused with CFPP_ERR_DIMS)
@@ -1646,6 +1712,19 @@ int launch_fused(const Plan& pl, const LayerParams& p, int grid, hipStream_t st)
 }
 bool fused_fits(const Plan& pl, const LayerParams& p, int grid) {
 #define X(a, b) if (pl.nch == a && pl.cpd == b) return fused_fits_t<a, b>(p, grid);
+    CFPP_SHAPE_CASES(X)
+#undef X
+    return false;
+}
+// `p0` is the first entry of `table` (device memory), on the host
+int launch_fused_stack(const Plan& pl, const LayerParams& p0, const LayerParams* table, int n_layers, int grid, hipStream_t st) {
+#define X(a, b) if (pl.nch == a && pl.cpd == b) return launch_fused_stack_t<a, b>(p0, table, n_layers, grid, st);
+    CFPP_SHAPE_CASES(X)
+#undef X
+    return CFPP_ERR_DIMS;
+}
+bool fused_stack_fits(const Plan& pl, const LayerParams& p, int grid) {
+#define X(a, b) if (pl.nch == a && pl.cpd == b) return fused_stack_fits_t<a, b>(p, grid);
     CFPP_SHAPE_CASES(X)
 #undef X
     return false;
@@ -2503,6 +2582,10 @@ struct cfpp_neox_stack {
     int* best_idx = nullptr;
     int* history = nullptr;
     int hist_cap = 0;
+    // fused mode, when the device holds the whole grid: the layers' parameters in device memory, for the one launch that
+    // runs all of them (null: one launch per layer)
+    LayerParams* table = nullptr;
+    LayerParams first{};          // table[0], on the host
     void* ws = nullptr;
     size_t ws_bytes = 0;
     // the device-resident position changes only through set_state and the steps, all of which pass through the host:
@@ -2530,15 +2613,51 @@ cfpp_neox_io stack_layer_io(const cfpp_neox_stack* s, int l) {
     io.max_seq_len = s->desc.cache_rows;
     return io;
 }
-int stack_enqueue_layer(cfpp_neox_stack* s, int l, hipStream_t st) {
+int stack_layer_params(const cfpp_neox_stack* s, int l, LayerParams* p, Plan* pl) {
     const cfpp_neox_io io = stack_layer_io(s, l);
-    LayerParams p;
-    Plan pl;
-    int rc = fill_params(&s->desc.dims, &s->layers[l], &io, s->ws, s->ws_bytes, true, true, &p, &pl);
+    const int rc = fill_params(&s->desc.dims, &s->layers[l], &io, s->ws, s->ws_bytes, true, true, p, pl);
     if (rc) return rc;
     // launch tags from the stack's step counter: no launch has to publish a generation for the next one
-    p.tag_src = s->state + 3; p.tag_mul = s->desc.n_layers; p.tag_add = l;
+    p->tag_src = s->state + 3; p->tag_mul = s->desc.n_layers; p->tag_add = l;
+    return CFPP_OK;
+}
+int stack_enqueue_layer(cfpp_neox_stack* s, int l, hipStream_t st) {
+    LayerParams p;
+    Plan pl;
+    const int rc = stack_layer_params(s, l, &p, &pl);
+    if (rc) return rc;
+    const cfpp_neox_io io = stack_layer_io(s, l);
     return run_layer(pl, p, s->desc.mode, seq_hint_of(&io), st);
+}
+// all layers: one launch when the stack has its table, one per layer otherwise
+int stack_enqueue_layers(cfpp_neox_stack* s, hipStream_t st) {
+    if (s->table != nullptr) return launch_fused_stack(s->plan, s->first, s->table, s->desc.n_layers, fused_grid(), st);
+    for (int l = 0; l < s->desc.n_layers; ++l) {
+        const int rc = stack_enqueue_layer(s, l, st);
+        if (rc) return rc;
+    }
+    return CFPP_OK;
+}
+// Fills the table if the one launch for all layers can be used: fused mode, every attention wave with one item at
+// most, the whole grid co-resident.
+int stack_make_table(cfpp_neox_stack* s, LayerParams* dev_table) {
+#ifdef CFPP_TRACE
+    return CFPP_OK;     // phase timestamps are per layer launch
+#endif
+    if (s->desc.mode != CFPP_MODE_FUSED) return CFPP_OK;
+    std::vector<LayerParams> host(s->desc.n_layers);
+    Plan pl;
+    for (int l = 0; l < s->desc.n_layers; ++l)
+        if (stack_layer_params(s, l, &host[l], &pl) != CFPP_OK) return CFPP_OK;     // the steps report what is wrong
+    const int grid = fused_grid();
+    if (grid > kLayerFlagWgs || (long long)host[0].heads * (host[0].max_split + 1) > (long long)grid * kStreamers ||
+        !fused_stack_fits(pl, host[0], grid))
+        return CFPP_OK;
+    const hipError_t e = hipMemcpy(dev_table, host.data(), host.size() * sizeof(LayerParams), hipMemcpyHostToDevice);
+    if (e != hipSuccess) return (int)e;
+    s->first = host[0];
+    s->table = dev_table;
+    return CFPP_OK;
 }
 
 LmTail stack_tail(const cfpp_neox_stack* s) {
@@ -2549,10 +2668,8 @@ LmTail stack_tail(const cfpp_neox_stack* s) {
 // fetches the picked token's embedding row for the next step
 int stack_enqueue_step(cfpp_neox_stack* s, hipStream_t st) {
     const cfpp_neox_dims& d = s->desc.dims;
-    for (int l = 0; l < s->desc.n_layers; ++l) {
-        const int rc = stack_enqueue_layer(s, l, st);
-        if (rc) return rc;
-    }
+    const int rc = stack_enqueue_layers(s, st);
+    if (rc) return rc;
     return launch_lm_head(d.hidden, s->desc.vocab, d.eps, s->hidden[s->desc.n_layers & 1], s->desc.final_ln_w,
                           s->desc.final_ln_b, s->desc.lm_head, s->logits, stack_tail(s), s->grid, st);
 }
@@ -2583,6 +2700,7 @@ int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out) {
     auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
     const size_t o_state = take(64), o_h0 = take((size_t)d.hidden * 2), o_h1 = take((size_t)d.hidden * 2);
     const size_t o_x0 = take((size_t)d.hidden * 2);
+    const size_t o_table = take((size_t)desc->n_layers * sizeof(LayerParams));
     const size_t o_k = take((size_t)d.hidden * 2), o_v = take((size_t)d.hidden * 2);
     const size_t o_logits = take((size_t)desc->vocab * 4);
     const size_t o_bv = take((size_t)s->grid * 4), o_bi = take((size_t)s->grid * 4);
@@ -2610,6 +2728,7 @@ int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out) {
     e = hipGetLastError();
     if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
     if (e != hipSuccess) { (void)hipFree(s->slab); delete s; return (int)e; }
+    if ((rc = stack_make_table(s, reinterpret_cast<LayerParams*>(s->slab + o_table)))) { (void)hipFree(s->slab); delete s; return rc; }
     *out = s;
     return CFPP_OK;
 }
@@ -2647,6 +2766,11 @@ int cfpp_stack_step(cfpp_neox_stack* s, void* stream) {
     rc = stack_enqueue_step(s, reinterpret_cast<hipStream_t>(stream));
     if (!rc) stack_advance(s, 1);
     return rc;
+}
+
+int cfpp_stack_layers_per_launch(const cfpp_neox_stack* s) {
+    if (!s) return CFPP_ERR_NULL;
+    return s->table != nullptr ? s->desc.n_layers : 1;
 }
 
 int cfpp_stack_check(cfpp_neox_stack* s, void* stream) {
@@ -2694,17 +2818,19 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
     const int L = s->desc.n_layers;
     std::vector<hipEvent_t> ev(L + 3);
     for (auto& e : ev) CFPP_HIP(hipEventCreate(&e));
-    // fused mode: one kernel per layer, timed from its own start to its own end; split mode (three kernels per layer):
-    // stream events between the layers, which include the launch gaps
-    bool fused = false;
-    if (s->desc.mode == CFPP_MODE_FUSED && s->desc.dims.heads <= fused_grid() * kStreamers) {
+    // fused mode: one kernel per layer, timed from its own start to its own end (with all layers in one launch: that
+    // launch, and every layer is reported as its share of it); split mode (three kernels per layer): stream events
+    // between the layers, which include the launch gaps
+    const bool chain = s->table != nullptr;
+    bool fused = chain;
+    if (!chain && s->desc.mode == CFPP_MODE_FUSED && s->desc.dims.heads <= fused_grid() * kStreamers) {
         const cfpp_neox_io io0 = stack_layer_io(s, 0);
         LayerParams p0;
         Plan pl0;
         if (fill_params(&s->desc.dims, &s->layers[0], &io0, s->ws, s->ws_bytes, true, true, &p0, &pl0) == CFPP_OK)
             fused = fused_fits(pl0, p0, fused_grid());
     }
-    std::vector<KernelEvents> kev(fused ? L : 0);
+    std::vector<KernelEvents> kev(chain ? 1 : (fused ? L : 0));
     for (auto& k : kev) {
         CFPP_HIP(hipEventCreate(&k.start));
         CFPP_HIP(hipEventCreate(&k.stop));
@@ -2713,7 +2839,12 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
     {
         const cfpp_neox_dims& d = s->desc.dims;
         CFPP_HIP(hipEventRecord(ev[L + 2], st));     // start of the step
-        for (int l = 0; l < L && !rc; ++l) {
+        if (chain) {
+            tl_kernel_events = &kev[0];
+            rc = stack_enqueue_layers(s, st);
+            tl_kernel_events = nullptr;
+        }
+        for (int l = 0; l < L && !rc && !chain; ++l) {
             CFPP_HIP(hipEventRecord(ev[l], st));
             if (fused) tl_kernel_events = &kev[l];
             rc = stack_enqueue_layer(s, l, st);
@@ -2731,9 +2862,12 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
     CFPP_HIP(hipEventRecord(end, st));
     CFPP_HIP(hipEventSynchronize(end));
     if (!rc) {
+        float all = 0.f;
+        if (chain) CFPP_HIP(hipEventElapsedTime(&all, kev[0].start, kev[0].stop));
         for (int l = 0; l < L; ++l) {
-            float ms = 0.f;
-            if (fused) CFPP_HIP(hipEventElapsedTime(&ms, kev[l].start, kev[l].stop));
+            float ms = all / (float)L;
+            if (chain) {}
+            else if (fused) CFPP_HIP(hipEventElapsedTime(&ms, kev[l].start, kev[l].stop));
             else CFPP_HIP(hipEventElapsedTime(&ms, ev[l], ev[l + 1]));
             if (layer_ms) layer_ms[l] = ms;
         }

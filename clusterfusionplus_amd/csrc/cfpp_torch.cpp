@@ -718,6 +718,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
             c10::hip::HIPGuardMasqueradingAsCUDA guard(s.device);
             check_rc(cfpp_stack_graph_steps(s.s, (int32_t)n, cur_stream()), "graph_steps");
         })
+        .def("layers_per_launch", [](PyStack& s) { return (int64_t)cfpp_stack_layers_per_launch(s.s); })
         .def("profile_step", [](PyStack& s) {
             // (per-layer ms list, lm head ms, whole-step ms) of one eager step timed with HIP events
             c10::hip::HIPGuardMasqueradingAsCUDA guard(s.device);

@@ -188,8 +188,15 @@ class NeoxDecoder:
         self._stack.graph_steps(int(n))
 
     def profile_step(self):
-        """One eager step with HIP events around every layer launch: (layer_ms list, lm_head_ms, step_ms)."""
+        """One eager step with HIP events around every layer launch: (layer_ms list, lm_head_ms, step_ms).  When one
+        launch runs all layers (`layers_per_launch`), every entry of the list is that launch's duration / n_layers."""
         return self._stack.profile_step()
+
+    @property
+    def layers_per_launch(self) -> int:
+        """Decoder layers per launch of a step: all of them when the stack runs the model's layers in one launch (fused
+        mode on a device that holds the whole grid), else 1."""
+        return int(self._stack.layers_per_launch())
 
     @property
     def logits(self) -> torch.Tensor:

@@ -326,13 +326,19 @@ int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out);
 int cfpp_stack_set_state(cfpp_neox_stack* s, int32_t token, int32_t seq_len, void* stream);
 /* One decode step launched eagerly: consumes (token, seq_len), appends K/V rows, writes logits,
  * then stores argmax as the new token and seq_len+1 and fetches the new token's embedding row (the LM head
- * launch does all of that: a step is n_layers + 1 launches in fused mode). */
+ * launch does all of that: a step is n_layers + 1 launches in fused mode, or 2 when one launch runs all layers,
+ * see cfpp_stack_layers_per_launch). */
 int cfpp_stack_step(cfpp_neox_stack* s, void* stream);
 /* Captures one step into a hipGraph (first call) and replays it `n_steps` times on `stream`. */
 int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream);
+/* Decoder layers that one launch of a step runs: n_layers when the stack runs all of them in a single launch (fused
+ * mode, the whole grid co-resident, a hidden size of whole 512-column chunks: the layers then hand their rows over inside
+ * the launch), 1 when every layer is a launch (or three, in split mode) of its own.  Fixed at creation. */
+int cfpp_stack_layers_per_launch(const cfpp_neox_stack* s);
 /* One eager decode step with a HIP event before and after every layer launch and the LM head, on
  * `stream`; synchronises.  layer_ms[n_layers], *lm_head_ms and *total_ms (whole step) receive elapsed
- * milliseconds.  For measurement; advances the state like cfpp_stack_step. */
+ * milliseconds (when one launch runs all layers, every layer_ms is that launch's duration / n_layers).  For
+ * measurement; advances the state like cfpp_stack_step. */
 int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, float* lm_head_ms, float* total_ms);
 /* Device pointers for inspection (read only: the token is changed through cfpp_stack_set_state, which also
  * fetches its embedding row): logits fp32 [vocab], hidden fp16 [H] after the last layer,

@@ -152,6 +152,8 @@ def test_stack_decode_matches_oracle(cf, model, mode):
     g_layers = [{n: t.to(dev) for n, t in w.items()} for w in layers]
     g_k, g_v = [t.to(dev) for t in kcs], [t.to(dev) for t in vcs]
     dec = pkg.NeoxDecoder(cfg, g_layers, embed.to(dev), fw.to(dev), fb.to(dev), lm.to(dev), g_k, g_v, mode=mode)
+    # fused mode runs the model's layers in one launch on a device that holds the whole grid; split mode never does
+    assert dec.layers_per_launch == (L if mode == "fused" else 1)
     tok = 17
     dec.set_state(tok, S)
     o_k, o_v = [t.clone() for t in kcs], [t.clone() for t in vcs]
@@ -179,6 +181,44 @@ def test_stack_decode_matches_oracle(cf, model, mode):
         tok = st[0]
         seq += 1
     assert len(dec.generated()) == 4
+
+
+@pytest.mark.parametrize("model,L", [("pythia_2b8", 1), ("pythia_2b8", 2), ("pythia_6b9", 5), ("pythia_160m", 3)])
+def test_layers_in_one_launch_equal_layers_in_launches_of_their_own(cf, model, L):
+    """The launch that runs all layers of a stack hands rows from layer to layer inside the launch; the per-stage launches
+    (split mode) hand them over at launch boundaries.  Same arithmetic: logits, hidden state, picks and cache rows must be
+    equal bit for bit, for one layer (no hand-over), two, and more, over several tokens (eager, then graph replays)."""
+    import clusterfusionplus_amd as pkg
+    dims = MODELS[model] if model in MODELS else O.NeoxDims(hidden=768, heads=12, head_dim=64, rotary_dim=16, ffn=3072)
+    V, rows, S, N = 500, 40, 9, 5
+    print(f"\ncase one launch == per stage, {model} L={L}", flush=True)
+    layers, embed, fw, fb, lm, kcs, vcs = _tiny_stack(L, V, rows, S, dims)
+    dev = "cuda:0"
+    cfg = pkg.NeoxConfig(dims.hidden, dims.heads, dims.head_dim, dims.rotary_dim, dims.ffn, L, V)
+    g_layers = [{n: t.to(dev) for n, t in w.items()} for w in layers]
+    out = {}
+    for mode in ("fused", "split"):
+        g_k, g_v = [t.to(dev) for t in kcs], [t.to(dev) for t in vcs]
+        dec = pkg.NeoxDecoder(cfg, g_layers, embed.to(dev), fw.to(dev), fb.to(dev), lm.to(dev), g_k, g_v, mode=mode)
+        if mode == "fused":
+            # hidden sizes that are not whole 512-column chunks (768) keep one launch per layer
+            assert dec.layers_per_launch == (L if dims.hidden % 512 == 0 else 1)
+        dec.set_state(3, S)
+        seen = []
+        for step in range(N):
+            if step == 0:
+                dec.step()
+            else:
+                dec.graph_steps(1)
+            torch.cuda.synchronize()
+            seen.append((dec.logits.clone(), dec.hidden.clone()))
+        dec.check()
+        out[mode] = (seen, dec.generated(), [t.clone() for t in g_k], [t.clone() for t in g_v])
+    assert out["fused"][1] == out["split"][1]
+    for (la, ha), (lb, hb) in zip(out["fused"][0], out["split"][0]):
+        assert torch.equal(la, lb) and torch.equal(ha, hb)
+    for a, b in zip(out["fused"][2] + out["fused"][3], out["split"][2] + out["split"][3]):
+        assert torch.equal(a, b)
 
 
 def test_lm_head_matches_torch(cf):
