@@ -353,12 +353,22 @@ __device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, c
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
+constexpr int kLayerFlagWgs = kEventGroups * kMailboxInts;
+// (One 16-byte load per lane that goes past the caches like an agent-scope atomic load, but as one request per 64-byte
+// line for the wave instead of two per lane: a buffer load with the sc1 bit.)
+__device__ __forceinline__ bool flags_all_set(const int* flags, int nwg, int tag, int lane) {
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(flags), 0, kLayerFlagWgs * 4, 0x00020000);
+    const u32x4 f = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane * 16, 0, 16);
+    const int i = lane * 4;
+    const bool ok = (i >= nwg || (int)(f.x - (uint32_t)tag) >= 0) && (i + 1 >= nwg || (int)(f.y - (uint32_t)tag) >= 0) &&
+                    (i + 2 >= nwg || (int)(f.z - (uint32_t)tag) >= 0) && (i + 3 >= nwg || (int)(f.w - (uint32_t)tag) >= 0);
+    return __builtin_amdgcn_ballot_w64(!ok) == 0;
+}
 // The hand-over between two layers of one launch: every workgroup has its own flag word (the words are the group
 // counters of kBarExit, which such a launch does not count in: kLayerFlagWgs workgroups at most) and stores its
 // layer's tag there once its output rows are in memory; a waiting wave reads all the words with one load per lane
 // until none is behind.  No counter has to be carried through the memory side's atomic units on the way from the last
 // row stored to the first row read: two round trips less than an event.
-constexpr int kLayerFlagWgs = kEventGroups * kMailboxInts;
 __device__ __forceinline__ void layer_done_post(int* grp, int wg, int tag, int lane) {
     drain_memory_ops();
     if (lane == 0) st_agent(reinterpret_cast<uint32_t*>(group_counter(grp, kBarExit, 0)) + wg, (uint32_t)tag);
@@ -366,12 +376,7 @@ __device__ __forceinline__ void layer_done_post(int* grp, int wg, int tag, int l
 __device__ __forceinline__ void layer_done_wait(int* grp, int nwg, int tag, const StatusSink& status, int lane) {
     const int* flags = group_counter(grp, kBarExit, 0);
     int spins = 0;
-    for (;;) {
-        const u32x4 f = ld_agent16(flags + lane * 4);
-        const int i = lane * 4;
-        const bool ok = (i >= nwg || (int)(f.x - (uint32_t)tag) >= 0) && (i + 1 >= nwg || (int)(f.y - (uint32_t)tag) >= 0) &&
-                        (i + 2 >= nwg || (int)(f.z - (uint32_t)tag) >= 0) && (i + 3 >= nwg || (int)(f.w - (uint32_t)tag) >= 0);
-        if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+    while (!flags_all_set(flags, nwg, tag, lane)) {
         __builtin_amdgcn_s_sleep(2);
         if (++spins > kSpinLimit) {
             if (lane == 0) raise_status(status, kStatusSpin);
