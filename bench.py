@@ -2,11 +2,13 @@
 """Benchmark of the whole-model decode step (TPOT) on one MI355X.
 
 A "step" is one generated token: embedding row -> 32 fused decoder layers -> final LayerNorm ->
-LM head -> argmax, replayed from one captured hipGraph, batch 1, fp16 weights (random init,
-synthetic) with fp32 accumulation, KV caches pre-filled to the given context.
+LM head -> argmax (two launches: all layers, then the LM head with the pick and the next embedding row),
+replayed from one captured hipGraph, batch 1, fp16 weights (random init, synthetic) with fp32
+accumulation, KV caches pre-filled to the given context.
 
 Prints ONE JSON line (last line of stdout).  `value` is ms per token (TPOT); `roofline` prices the
-dominant kernel (the fused decoder-layer kernel) against the 8 TB/s HBM peak using algorithmic bytes
+dominant kernel (the launch that runs the decoder layers: k_fused_stack, all layers in one launch, or
+k_fused, one layer, with --mode fused_layers) against the 8 TB/s HBM peak using algorithmic bytes
 (weights + small vectors + KV rows [0,S), read once) over its HIP-event-timed launch duration;
 `cpu_baseline` is the HuggingFace GPTNeoXLayer fp32 path timed on this box's host cores on a bounded
 sample (reported, not a target).
@@ -24,13 +26,13 @@ HBM_PEAK_GBPS = 8000.0
 
 
 
-def recorded_traffic(model, ctx):
+def recorded_traffic(model, ctx, kernel="k_fused"):
     """HBM bytes per launch of the fused layer kernel (fetched + written) as recorded in the committed hardware-counter
     summary of this workload (two `rocprofv3 --pmc` runs of this script, FETCH_SIZE and WRITE_SIZE, scaled by the
     256 MiB calibration copy): the number on the summary's `traffic_bytes_per_launch:` line and the file it came from,
     or (None, None) when no summary exists for the workload.  A counter run cannot be part of a timed run; the
     summary states the command and the commit it was taken at."""
-    rel = os.path.join("profiles", f"k_fused_{model}_ctx{ctx}_hbm_traffic.txt")
+    rel = os.path.join("profiles", f"{kernel}_{model}_ctx{ctx}_hbm_traffic.txt")
     try:
         with open(os.path.join(ROOT, rel)) as f:
             for line in f:
@@ -519,7 +521,9 @@ def main():
     ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8", "llama2_7b_layer", "llama2_7b_batch"])
     ap.add_argument("--batch", type=int, default=16, help="sequences per call (llama2_7b_batch only)")
     ap.add_argument("--ctx", type=int, default=2048, help="KV-cache rows already filled when the timed region starts")
-    ap.add_argument("--mode", default="fused", choices=["fused", "split"])
+    ap.add_argument("--mode", default="fused", choices=["fused", "split", "fused_layers"],
+                    help="fused: one launch per layer, or one for all layers where the device holds the whole grid; "
+                         "fused_layers: one launch per layer in any case; split: one launch per stage")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-also", dest="also", action="store_false",
                     help="skip the context sweep, the drop-in per-layer loop and the short measurements of the other configurations")
@@ -590,7 +594,6 @@ def main():
     ev_ms = e0.elapsed_time(e1)
     tpot = wall_ms / K
     dec.check()                       # raises if any launch of the run raised a device-side failure flag
-    traffic, traffic_source = recorded_traffic(args.model, args.ctx) if args.mode == "fused" else (None, None)
 
     S_mid = args.ctx + W + K // 2
     sb = step_bytes(cfg, S_mid)
@@ -602,7 +605,10 @@ def main():
     if per_launch > 1:
         kernel_name = f"k_fused_stack (all {per_launch} decoder layers in one launch)"
     else:
-        kernel_name = "k_fused (one decoder layer)" if args.mode == "fused" else "stage A+B+C kernels (one decoder layer)"
+        kernel_name = "k_fused (one decoder layer)" if args.mode != "split" else "stage A+B+C kernels (one decoder layer)"
+    traffic, traffic_source = (None, None)
+    if args.mode != "split":
+        traffic, traffic_source = recorded_traffic(args.model, args.ctx, "k_fused_stack" if per_launch > 1 else "k_fused")
     result = {
         "metric": "tpot_ms", "value": round(tpot, 4), "unit": "ms/token", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(tpot, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,

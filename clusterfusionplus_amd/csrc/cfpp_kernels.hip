@@ -2683,7 +2683,7 @@ int cfpp_stack_create(const cfpp_neox_stack_desc* desc, cfpp_neox_stack** out) {
     if (!desc->layers || !desc->embed || !desc->final_ln_w || !desc->final_ln_b || !desc->lm_head || !desc->k_caches ||
         !desc->v_caches || !desc->rope_cos || !desc->rope_sin)
         return CFPP_ERR_NULL;
-    if (desc->mode != CFPP_MODE_FUSED && desc->mode != CFPP_MODE_SPLIT) return CFPP_ERR_MODE;
+    if (desc->mode != CFPP_MODE_FUSED && desc->mode != CFPP_MODE_SPLIT && desc->mode != CFPP_MODE_FUSED_LAYERS) return CFPP_ERR_MODE;
     cfpp_neox_stack* s = new cfpp_neox_stack();
     s->desc = *desc;
     s->layers.assign(desc->layers, desc->layers + desc->n_layers);
@@ -2823,7 +2823,7 @@ int cfpp_stack_profile_step(cfpp_neox_stack* s, void* stream, float* layer_ms, f
     // between the layers, which include the launch gaps
     const bool chain = s->table != nullptr;
     bool fused = chain;
-    if (!chain && s->desc.mode == CFPP_MODE_FUSED && s->desc.dims.heads <= fused_grid() * kStreamers) {
+    if (!chain && s->desc.mode != CFPP_MODE_SPLIT && s->desc.dims.heads <= fused_grid() * kStreamers) {
         const cfpp_neox_io io0 = stack_layer_io(s, 0);
         LayerParams p0;
         Plan pl0;

@@ -162,7 +162,7 @@ class NeoxDecoder:
         packed = [[w[k].reshape(-1) if w[k].dim() == 1 else w[k] for k in layer_tensor_order] for w in layers]
         self._stack = native.NeoxStack(cfg.hidden, cfg.heads, cfg.head_dim, cfg.rotary_dim, cfg.ffn, cfg.eps,
                                        packed, embed, final_ln_w, final_ln_b, lm_head, list(k_caches), list(v_caches),
-                                       self.cos, self.sin, {"fused": 0, "split": 1}[mode])
+                                       self.cos, self.sin, {"fused": 0, "split": 1, "fused_layers": 2}[mode])
 
     @classmethod
     def from_hf(cls, hf_model, past_key_values, max_rows: int, device="cuda", mode: str = "fused"):

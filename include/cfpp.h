@@ -99,7 +99,9 @@ typedef struct cfpp_neox_io {
 
 typedef enum cfpp_mode {
     CFPP_MODE_FUSED = 0,     /* one persistent launch with device-wide barriers between the stages */
-    CFPP_MODE_SPLIT = 1      /* one plain launch per stage; the kernel boundary is the barrier */
+    CFPP_MODE_SPLIT = 1,     /* one plain launch per stage; the kernel boundary is the barrier */
+    CFPP_MODE_FUSED_LAYERS = 2   /* cfpp_stack_* only: CFPP_MODE_FUSED with every layer a launch of its own, also where one
+                                  * launch could run all layers (cfpp_stack_layers_per_launch); for comparison and profiling */
 } cfpp_mode;
 
 const char* cfpp_status_str(int status);
@@ -313,7 +315,7 @@ typedef struct cfpp_neox_stack_desc {
     int32_t cache_rows;
     const float* rope_cos;             /* [cache_rows, rotary_dim] fp32 table indexed by position */
     const float* rope_sin;
-    int32_t mode;                      /* cfpp_mode used for every layer */
+    int32_t mode;                      /* cfpp_mode used for every layer (CFPP_MODE_FUSED_LAYERS allowed) */
 } cfpp_neox_stack_desc;
 
 typedef struct cfpp_neox_stack cfpp_neox_stack;   /* opaque */

@@ -185,8 +185,8 @@ def test_stack_decode_matches_oracle(cf, model, mode):
 
 @pytest.mark.parametrize("model,L", [("pythia_2b8", 1), ("pythia_2b8", 2), ("pythia_6b9", 5), ("pythia_160m", 3)])
 def test_layers_in_one_launch_equal_layers_in_launches_of_their_own(cf, model, L):
-    """The launch that runs all layers of a stack hands rows from layer to layer inside the launch; the per-stage launches
-    (split mode) hand them over at launch boundaries.  Same arithmetic: logits, hidden state, picks and cache rows must be
+    """The launch that runs all layers of a stack hands rows from layer to layer inside the launch; one launch per layer
+    (fused_layers) and the per-stage launches (split mode) hand them over at launch boundaries.  Same arithmetic: logits, hidden state, picks and cache rows must be
     equal bit for bit, for one layer (no hand-over), two, and more, over several tokens (eager, then graph replays)."""
     import clusterfusionplus_amd as pkg
     dims = MODELS[model] if model in MODELS else O.NeoxDims(hidden=768, heads=12, head_dim=64, rotary_dim=16, ffn=3072)
@@ -197,12 +197,14 @@ def test_layers_in_one_launch_equal_layers_in_launches_of_their_own(cf, model, L
     cfg = pkg.NeoxConfig(dims.hidden, dims.heads, dims.head_dim, dims.rotary_dim, dims.ffn, L, V)
     g_layers = [{n: t.to(dev) for n, t in w.items()} for w in layers]
     out = {}
-    for mode in ("fused", "split"):
+    for mode in ("fused", "fused_layers", "split"):
         g_k, g_v = [t.to(dev) for t in kcs], [t.to(dev) for t in vcs]
         dec = pkg.NeoxDecoder(cfg, g_layers, embed.to(dev), fw.to(dev), fb.to(dev), lm.to(dev), g_k, g_v, mode=mode)
         if mode == "fused":
             # hidden sizes that are not whole 512-column chunks (768) keep one launch per layer
             assert dec.layers_per_launch == (L if dims.hidden % 512 == 0 else 1)
+        else:
+            assert dec.layers_per_launch == 1
         dec.set_state(3, S)
         seen = []
         for step in range(N):
@@ -214,11 +216,12 @@ def test_layers_in_one_launch_equal_layers_in_launches_of_their_own(cf, model, L
             seen.append((dec.logits.clone(), dec.hidden.clone()))
         dec.check()
         out[mode] = (seen, dec.generated(), [t.clone() for t in g_k], [t.clone() for t in g_v])
-    assert out["fused"][1] == out["split"][1]
-    for (la, ha), (lb, hb) in zip(out["fused"][0], out["split"][0]):
-        assert torch.equal(la, lb) and torch.equal(ha, hb)
-    for a, b in zip(out["fused"][2] + out["fused"][3], out["split"][2] + out["split"][3]):
-        assert torch.equal(a, b)
+    for other in ("fused_layers", "split"):
+        assert out["fused"][1] == out[other][1]
+        for (la, ha), (lb, hb) in zip(out["fused"][0], out[other][0]):
+            assert torch.equal(la, lb) and torch.equal(ha, hb)
+        for a, b in zip(out["fused"][2] + out["fused"][3], out[other][2] + out[other][3]):
+            assert torch.equal(a, b)
 
 
 def test_lm_head_matches_torch(cf):
