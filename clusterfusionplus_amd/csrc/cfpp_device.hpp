@@ -373,17 +373,21 @@ __device__ __forceinline__ void layer_done_post(int* grp, int wg, int tag, int l
     drain_memory_ops();
     if (lane == 0) st_agent(reinterpret_cast<uint32_t*>(group_counter(grp, kBarExit, 0)) + wg, (uint32_t)tag);
 }
-__device__ __forceinline__ void layer_done_wait(int* grp, int nwg, int tag, const StatusSink& status, int lane) {
+// (false: the wait expired; the status flag is raised)
+__device__ __forceinline__ bool layer_done_wait(int* grp, int nwg, int tag, const StatusSink& status, int lane) {
     const int* flags = group_counter(grp, kBarExit, 0);
     int spins = 0;
+    bool ok = true;
     while (!flags_all_set(flags, nwg, tag, lane)) {
         __builtin_amdgcn_s_sleep(2);
         if (++spins > kSpinLimit) {
             if (lane == 0) raise_status(status, kStatusSpin);
+            ok = false;
             break;
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    return ok;
 }
 
 __device__ __forceinline__ StatusSink status_sink(const LayerParams& p) { return StatusSink{p.bar + kBarStatus, p.host_status}; }

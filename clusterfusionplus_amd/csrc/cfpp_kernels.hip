@@ -345,7 +345,7 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_stage_c8(LayerParams p)
 // co-resident (the host launches one per compute unit); every wait is bounded.
 constexpr int kXcds = 8;      // chiplets (accelerator complex dies) of the device, each with its own L2
 constexpr long long kXcdGroupBytes = 3 << 19;     // 1.5 MB of the 4 MB
-struct FusedShared { int arrived[1 + kUpPhases]; };
+struct FusedShared { int arrived[1 + kUpPhases]; int give_up; };
 
 
 template <int NCH>
@@ -365,7 +365,7 @@ struct FusedLds {
 // of them have said so (layer_done_wait for the previous layer's tag, tag - 1), with the first weight tiles already
 // requested; `announce` makes it say so itself once its output rows are stored.  Rows that cross layers go past the caches.
 template <int NCH, int CPD, bool EX, bool BYX, bool CHAIN = false>
-__device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, FusedLds<NCH>& lds, bool wait_prev = false,
+__device__ __forceinline__ bool fused_layer(const LayerParams& p, int gen_word, FusedLds<NCH>& lds, bool wait_prev = false,
                                             bool announce = false) {
     FusedShared& q = lds.q;
     StageCShared& shc = lds.shc;
@@ -383,6 +383,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
     const StatusSink status = status_sink(p);
     const int seq_requested = seq_len_request(p);     // on its way before anything else
     if (thread <= kUpPhases) q.arrived[thread] = 0;
+    if (CHAIN && thread == kUpPhases + 1) q.give_up = 0;
     __syncthreads();
     trace_mark(p, 0);
     trace_value(p, 8, __builtin_amdgcn_s_getreg((3 << 11) | 20));   // XCC_ID: which XCD this workgroup runs on
@@ -415,7 +416,9 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
             // workgroups finish that layer.  One wave polls, the others wait for it at the barrier.
             if constexpr (decltype(with_tile)::value) qkv_prefetch<NCH, EX>(p, qw, lane, t0);
             if (wait_prev) {
-                if (wave == kFusedWaves - 1) layer_done_wait(p.grp, G, first_lane(gen_word) * p.tag_mul + p.tag_add, status, lane);
+                if (wave == kFusedWaves - 1 &&
+                    !layer_done_wait(p.grp, G, first_lane(gen_word) * p.tag_mul + p.tag_add, status, lane) && lane == 0)
+                    q.give_up = 1;
                 __syncthreads();
             }
             ln_coop_load<NCH, kFusedWaves, true, true>(own, norm_spec(p), wave, lane);
@@ -432,6 +435,10 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
     };
     if (qkv8 || wave < kStreamers) norm_phase(std::true_type{});
     else norm_phase(std::false_type{});
+    // A wait for the previous layer that expired (the status flag is raised: some workgroup is not running, which the
+    // host's co-residency check is there to exclude) ends the launch for this workgroup: every later wait would expire as
+    // well, a second at a time.  The workgroups that wait for this one give up at their own next layer.
+    if (CHAIN && wait_prev && q.give_up) return false;
     trace_mark(p, 1);
     // The launch tag and the sequence length were requested at the top of the kernel.  They are looked at (`resolve`)
     // only once a wave has used up its first weight tile: every load of a wave returns in order, so by then they are
@@ -593,6 +600,7 @@ __device__ __forceinline__ void fused_layer(const LayerParams& p, int gen_word, 
         const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1, tag, lane);
         if (last && lane == 0) __hip_atomic_store(p.bar + kBarGen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    return true;
 }
 
 // one layer, parameters in the kernel arguments
@@ -619,7 +627,7 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused_stack(const Layer
     const int gen_word = first_lane(counter_peek(((ConstLayerParams*)table)->tag_src));     // the same word for every layer
     for (int l = 0; l < n_layers; ++l) {
         const LayerParams& p = *(const LayerParams*)((ConstLayerParams*)table + l);
-        fused_layer<NCH, CPD, EX, BYX, true>(p, gen_word, lds, l > 0, l + 1 < n_layers);
+        if (!fused_layer<NCH, CPD, EX, BYX, true>(p, gen_word, lds, l > 0, l + 1 < n_layers)) break;
     }
 }
 
