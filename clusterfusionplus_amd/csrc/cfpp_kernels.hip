@@ -2594,6 +2594,10 @@ struct cfpp_neox_stack {
     // runs all of them (null: one launch per layer)
     LayerParams* table = nullptr;
     LayerParams first{};          // table[0], on the host
+#ifdef CFPP_TRACE
+    std::vector<LayerParams> host_table;     // profiling builds: the table is rewritten when the trace buffer changes
+    long long* table_trace = nullptr;
+#endif
     void* ws = nullptr;
     size_t ws_bytes = 0;
     // the device-resident position changes only through set_state and the steps, all of which pass through the host:
@@ -2639,6 +2643,16 @@ int stack_enqueue_layer(cfpp_neox_stack* s, int l, hipStream_t st) {
 }
 // all layers: one launch when the stack has its table, one per layer otherwise
 int stack_enqueue_layers(cfpp_neox_stack* s, hipStream_t st) {
+#ifdef CFPP_TRACE
+    // layer l stamps into its own [workgroups][waves][slots] block of the trace buffer
+    if (s->table != nullptr && s->table_trace != g_trace) {
+        for (size_t l = 0; l < s->host_table.size(); ++l)
+            s->host_table[l].trace = g_trace ? g_trace + l * ((size_t)kMaxGrid * kMaxWaves * kTraceSlots) : nullptr;
+        CFPP_HIP(hipStreamSynchronize(st));
+        CFPP_HIP(hipMemcpy(s->table, s->host_table.data(), s->host_table.size() * sizeof(LayerParams), hipMemcpyHostToDevice));
+        s->table_trace = g_trace;
+    }
+#endif
     if (s->table != nullptr) return launch_fused_stack(s->plan, s->first, s->table, s->desc.n_layers, fused_grid(), st);
     for (int l = 0; l < s->desc.n_layers; ++l) {
         const int rc = stack_enqueue_layer(s, l, st);
@@ -2649,9 +2663,6 @@ int stack_enqueue_layers(cfpp_neox_stack* s, hipStream_t st) {
 // Fills the table if the one launch for all layers can be used: fused mode, every attention wave with one item at
 // most, the whole grid co-resident.
 int stack_make_table(cfpp_neox_stack* s, LayerParams* dev_table) {
-#ifdef CFPP_TRACE
-    return CFPP_OK;     // phase timestamps are per layer launch
-#endif
     if (s->desc.mode != CFPP_MODE_FUSED) return CFPP_OK;
     std::vector<LayerParams> host(s->desc.n_layers);
     Plan pl;
@@ -2665,6 +2676,10 @@ int stack_make_table(cfpp_neox_stack* s, LayerParams* dev_table) {
     if (e != hipSuccess) return (int)e;
     s->first = host[0];
     s->table = dev_table;
+#ifdef CFPP_TRACE
+    s->host_table = host;
+    s->table_trace = host[0].trace;
+#endif
     return CFPP_OK;
 }
 

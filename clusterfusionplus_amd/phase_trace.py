@@ -9,6 +9,9 @@ package import would load the product library first):
 
     python -m clusterfusionplus_amd.build --trace-lib /tmp/libcfpp_trace.so
     python clusterfusionplus_amd/phase_trace.py --trace-lib /tmp/libcfpp_trace.so --model pythia_2b8 --ctx 1024
+
+With --stack the step goes through the launch that runs all layers of the model (the whole-model decoder's own path):
+the same table per layer of that launch, and the hand-over from layer to layer inside it.
 """
 import argparse
 import ctypes
@@ -65,6 +68,9 @@ def main():
     ap.add_argument("--model", default="pythia_6b9", choices=["pythia_6b9", "pythia_2b8", "llama2_7b_attention"])
     ap.add_argument("--ctx", type=int, default=2048)
     ap.add_argument("--raw", help="also save the raw timestamps of every layer ([layer][workgroup][wave][slot]) as .npy")
+    ap.add_argument("--stack", action="store_true",
+                    help="trace the launch that runs all layers of the model (one eager step): the phases of every layer, "
+                         "and how the rows pass from layer to layer inside the launch")
     a = ap.parse_args()
     load_trace_library(a.trace_lib)
     from clusterfusionplus_amd import PYTHIA_2B8, PYTHIA_6B9, debug_set_trace
@@ -78,6 +84,8 @@ def main():
         dec.step()
     torch.cuda.synchronize()
     lay, _lm, _tot = dec.profile_step()
+    if a.stack:
+        return stack_launch(a, dec, cfg, lay, dev)
     print(f"{a.model}, context {a.ctx}: fused layer kernel {np.median(lay) * 1e3:.1f} us (median of {len(lay)} layers, HIP events, "
           "profiling build)")
     # the trace buffer holds one launch: record the layers of one step one at a time through the per-layer op
@@ -100,6 +108,47 @@ def main():
     if a.raw:
         np.save(a.raw, np.stack(per_layer))
     report(per_layer[2:])
+    return 0
+
+
+def stack_launch(a, dec, cfg, lay, dev):
+    """One eager step through the launch that runs all layers; layer l stamps into block l of the trace buffer."""
+    from clusterfusionplus_amd import debug_set_trace
+    L = cfg.n_layers
+    if dec.layers_per_launch != L:
+        raise RuntimeError("this stack runs one launch per layer (see NeoxDecoder.layers_per_launch): nothing to trace with --stack")
+    print(f"{a.model}, context {a.ctx}: all {L} layers in one launch, {sum(lay) * 1e3:.0f} us = {np.mean(lay) * 1e3:.1f} us per layer "
+          "(HIP events, profiling build)")
+    block = 1024 * 16 * 16
+    tr = torch.zeros(L * block, dtype=torch.int64, device=dev)
+    debug_set_trace(tr)
+    dec.step()
+    torch.cuda.synchronize()
+    debug_set_trace(None)
+    dec.step()                       # (the table forgets the buffer before it is freed)
+    torch.cuda.synchronize()
+    raw = tr.cpu().numpy().reshape(L, 1024, 16, 16)[:, :256, :8].astype(np.float64)
+    if a.raw:
+        np.save(a.raw, raw)
+    report(list(raw[2:]))
+    # the hand-over: from the last output row of layer l to the norm of layer l + 1
+    def stamps(l, slot):
+        v = raw[l][:, :, slot]
+        return v[v > 0]
+    rows = []
+    for l in range(2, L - 1):
+        done = stamps(l, 10)                 # stage C done, per wave
+        end = done.max()
+        seen, norm, entry = stamps(l + 1, 14), stamps(l + 1, 1), stamps(l + 1, 0)
+        rows.append(((end - done.min()) / 100, (np.median(done) - end) / 100, (np.median(entry) - end) / 100, (entry.max() - end) / 100,
+                     (np.median(seen) - end) / 100, (seen.max() - end) / 100, (np.median(norm) - end) / 100, (norm.max() - end) / 100))
+    m = np.median(np.array(rows), axis=0)
+    print("hand-over between layers (us relative to the moment the last wave of layer l has stored its output rows; median over layers)")
+    print(f"  first wave of layer l done                                         {-m[0]:8.2f}")
+    print(f"  median wave of layer l done                                        {m[1]:8.2f}")
+    print(f"  layer l+1 entered (median / last wave)                             {m[2]:8.2f} {m[3]:8.2f}")
+    print(f"  layer l complete seen, input row requested (median / last wave)    {m[4]:8.2f} {m[5]:8.2f}")
+    print(f"  norm of layer l+1 done (median / last wave)                        {m[6]:8.2f} {m[7]:8.2f}")
     return 0
 
 
