@@ -354,8 +354,9 @@ __device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, c
 }
 
 constexpr int kLayerFlagWgs = kEventGroups * kMailboxInts;
-// (One 16-byte load per lane that goes past the caches like an agent-scope atomic load, but as one request per 64-byte
-// line for the wave instead of two per lane: a buffer load with the sc1 bit.)
+// (One 16-byte load per lane that goes past the caches like an agent-scope atomic load, as a single instruction: a buffer
+// load with the sc1 bit, cache policy 16.  The descriptor is a raw buffer over the kLayerFlagWgs words; 0x00020000 is the
+// data-format field of word 3 that gfx9 buffer descriptors of 32-bit elements carry.)
 __device__ __forceinline__ bool flags_all_set(const int* flags, int nwg, int tag, int lane) {
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(flags), 0, kLayerFlagWgs * 4, 0x00020000);
     const u32x4 f = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane * 16, 0, 16);

@@ -335,7 +335,8 @@ int cfpp_stack_step(cfpp_neox_stack* s, void* stream);
 int cfpp_stack_graph_steps(cfpp_neox_stack* s, int32_t n_steps, void* stream);
 /* Decoder layers that one launch of a step runs: n_layers when the stack runs all of them in a single launch (fused
  * mode, the whole grid co-resident, a hidden size of whole 512-column chunks: the layers then hand their rows over inside
- * the launch), 1 when every layer is a launch (or three, in split mode) of its own.  Fixed at creation. */
+ * the launch), 1 when every layer is a launch (or three, in split mode) of its own.  Fixed at creation.  CFPP_ERR_NULL
+ * (negative) for a null stack. */
 int cfpp_stack_layers_per_launch(const cfpp_neox_stack* s);
 /* One eager decode step with a HIP event before and after every layer launch and the LM head, on
  * `stream`; synchronises.  layer_ms[n_layers], *lm_head_ms and *total_ms (whole step) receive elapsed
