@@ -92,6 +92,7 @@ def test_one_launch_rule_and_device_status_without_a_gpu(lib):
     assert lib.cfpp_device_status(0) == 0 and lib.cfpp_device_status(1) == 0
     assert lib.cfpp_ctx_check(0, ctypes.c_int64(4242), None) == -5          # unknown context
     assert lib.cfpp_stack_check(None, None) == -1
+    assert lib.cfpp_stack_layers_per_launch(None) == -1
 
 
 class NeoxIo(ctypes.Structure):
