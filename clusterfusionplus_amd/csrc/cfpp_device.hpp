@@ -53,15 +53,15 @@ constexpr int kHeadCntStride = 16;     // ints between the arrival counters of t
 
 enum : int { kStatusSpin = 1, kStatusSeq = 2 };
 // Slots of LayerParams::bar.  The event counters reset themselves (the arrival that completes a count
-// stores zero); flags are not reset at all: a launch raises a flag by writing its tag, the launch
-// generation read from kBarGen plus one, and the last workgroup to leave stores that tag back.
+// stores zero); flags are not reset at all: a launch raises a flag by writing its tag, which no earlier
+// launch on the workspace has used (launch_generation below, or a counter of the caller's).
 enum BarSlot : int {
     kBarQkv = 0,                      // streaming waves that have written their QKV rows
     kBarUp = 1,                       // kBarUp + g: streaming waves that have written their MLP-up rows of phase g (kUpPhases slots)
     kBarHeads = kBarUp + kUpPhases,   // heads whose attention output is merged
-    kBarExit = kBarHeads + 1,         // workgroups that have finished
+    kBarExit = kBarHeads + 1,         // workgroups that have finished (only its group counters are used, see launch_generation)
     kBarStatus = kBarExit + 1,        // failure flags (kStatusSpin, kStatusSeq); never reset by the kernels
-    kBarGen = kBarStatus + 1          // launch generation
+    kBarGen = kBarStatus + 1          // (unused)
 };
 static_assert(kBarGen < 16, "the slots are the ints of one 64-byte line");
 
@@ -351,6 +351,30 @@ __device__ __forceinline__ void event_wait(const int* mbox, int slot, int tag, c
     }
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// The launch generation of a workspace: the number of workgroups that have ever finished a one-launch kernel on it,
+// kept in the kEventGroups group counters of kBarExit (never reset).  A workgroup that leaves adds one to the counter
+// of its group without waiting for the result (launch_generation_leave); the next launch starts after this one has
+// completed, reads the counters (one per lane, launch_generation_request) and takes their sum + 1 as its tag
+// (launch_generation_tag): larger than any tag before it.  Within a launch every workgroup sees the same sum: none can
+// leave before all of them have passed the device-wide events, and they read the counters first thing.  (Publishing a
+// generation word from the last workgroup to leave instead took that workgroup two dependent atomics, with their
+// return values, at the very end of every launch.)
+__device__ __forceinline__ int launch_generation_request(int* grp, int lane) {
+    return counter_peek(group_counter(grp, kBarExit, lane % kEventGroups));
+}
+__device__ __forceinline__ int launch_generation_tag(int requested, int lane) {
+    int v = lane < kEventGroups ? requested : 0;
+    static_assert(kEventGroups == 16, "the sum below runs over sixteen lanes");
+    v += __shfl_xor(v, 8, kWave);
+    v += __shfl_xor(v, 4, kWave);
+    v += __shfl_xor(v, 2, kWave);
+    v += __shfl_xor(v, 1, kWave);
+    return __builtin_amdgcn_readfirstlane(v) + 1;
+}
+__device__ __forceinline__ void launch_generation_leave(int* grp, int wg, int lane) {
+    if (lane == 0) __hip_atomic_fetch_add(group_counter(grp, kBarExit, wg % kEventGroups), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 constexpr int kLayerFlagWgs = kEventGroups * kMailboxInts;

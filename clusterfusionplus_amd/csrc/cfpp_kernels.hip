@@ -229,7 +229,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_up(LayerParams p) {
 // The whole gated MLP block in one launch: norm -> gate/up pairs in kUpPhases phases (a wave owns a contiguous range
 // of pairs of every phase; event kBarUp + g after phase g) -> down rows of stage C, which start on phase g of the
 // intermediate as soon as its event is complete, with their first weight tiles requested before the wait.  One
-// workgroup per compute unit, all co-resident; launch tag from the generation word, published again at the end.
+// workgroup per compute unit, all co-resident; launch tag from the workspace's launch generation.
 template <int NCH, int CPD, bool EX>
 __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
     touch_kernel_arguments<kLayerKernargBytes>();
@@ -237,8 +237,8 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
     __shared__ LnShared<NCH> lns;
     __shared__ StageCShared shc;
     __shared__ int arrived[kUpPhases];
-    const int gen = counter_peek(p.bar + kBarGen);
     const int lane = threadIdx.x & 63, wave = first_lane(threadIdx.x >> 6);
+    const int gen = launch_generation_request(p.grp, lane);
     const int G = gridDim.x, b = blockIdx.x;
     const int gw = b * kStreamers + wave, nw = G * kStreamers;
     const StatusSink status = status_sink(p);
@@ -258,7 +258,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
     RowTile<NCH, 2> t0;
     prefetch_row_tile<NCH, 2, EX>(t0, p.w_up, p.H, first, F, 2 * F, count, lane);
     ln_coop_finish<NCH, kStreamers, false>(own, norm_spec(p), lns, wave, lane);
-    const int tag = first_lane(gen) + 1;
+    const int tag = launch_generation_tag(gen, lane);
     half2_t xr[NCH][4];
     ln_fetch<NCH>(lns, 0, lane, xr);
 #pragma unroll
@@ -280,10 +280,7 @@ __global__ __launch_bounds__(kStreamers * 64) void k_gated_mlp(LayerParams p) {
     const StageC c = make_stage_c(p);
     stage_c_rows<NCH, CPD>(c, b, G, shc, true, wave, wave, kStreamers, lane,
                            [&](int g) { event_wait(p.mbox, kBarUp + g, tag, status); }, [] {});
-    if (wave == 0) {
-        const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1, tag);
-        if (last && lane == 0) __hip_atomic_store(p.bar + kBarGen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    if (wave == 0) launch_generation_leave(p.grp, b, lane);
 }
 
 // one (head, split) item per wave
@@ -340,7 +337,7 @@ __global__ __launch_bounds__(2 * kStreamers * 64) void k_stage_c8(LayerParams p)
 //                   trips; it and the O projection run beside the MLP-up / MLP-down streaming instead of in
 //                   front of it.
 //   all waves:      row reduction in LDS, bias, residual.
-// Nothing is reset at the end: counters zero themselves and flags carry a launch tag (from the generation word of the
+// Nothing is reset at the end: counters zero themselves and flags carry a launch tag (from the launch generation of the
 // workspace, or from the caller's step counter in the whole-model decoder).  All workgroups must be
 // co-resident (the host launches one per compute unit); every wait is bounded.
 constexpr int kXcds = 8;      // chiplets (accelerator complex dies) of the device, each with its own L2
@@ -463,7 +460,7 @@ __device__ __forceinline__ bool fused_layer(const LayerParams& p, int gen_word, 
     // the count to the device-wide counters.  (Not at the QKV event: the attention waves wait for that one, and
     // an arrival that goes through another wave reaches them later.)
     auto resolve = [&]() {
-        tag = first_lane(gen_word) * (p.tag_src != nullptr ? p.tag_mul : 1) + (p.tag_src != nullptr ? p.tag_add : 0) + 1;
+        tag = p.tag_src != nullptr ? first_lane(gen_word) * p.tag_mul + p.tag_add + 1 : launch_generation_tag(gen_word, lane);
         sl = seq_len_check(p, first_lane(seq_requested));
         nsplit = effective_split(p, sl.S);
         per_head = items_per_head(nsplit);
@@ -596,9 +593,7 @@ __device__ __forceinline__ bool fused_layer(const LayerParams& p, int gen_word, 
         // the wave that stored this workgroup's output rows raises the workgroup's flag for the next layer
         if (wave == 0 && announce) layer_done_post(p.grp, b, tag, lane);
     } else if (wave == 0 && p.tag_src == nullptr) {
-        // the last workgroup to leave publishes the new generation: the flags of this launch turn stale
-        const bool last = event_arrive(p.bar, p.grp, nullptr, kBarExit, G, nullptr, 1, tag, lane);
-        if (last && lane == 0) __hip_atomic_store(p.bar + kBarGen, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        launch_generation_leave(p.grp, b, lane);      // the flags of this launch turn stale for the next one
     }
     return true;
 }
@@ -608,11 +603,12 @@ template <int NCH, int CPD, bool EX, bool BYX>
 __global__ __launch_bounds__(2 * kStreamers * 64) void k_fused(LayerParams p) {
     touch_kernel_arguments<kLayerKernargBytes>();
     __shared__ FusedLds<NCH> lds;
-    // the flag value of this launch is gen + 1: requested first, needed at the first event.  It comes from the
-    // generation the previous launch on this workspace published, or from a counter that the caller advances
-    // between launches (a whole-model step: step counter x layers + layer), which saves the publishing.
+    // what the flag value (tag) of this launch derives from: requested first, needed at the first event.  The workspace's
+    // launch generation (launch_generation_request: a counter per lane), or a counter that the caller advances between
+    // launches (a whole-model step: step counter x layers + layer).
     // (a vector load; nothing looks at the value until the wave has used up its first weight tile)
-    const int gen_word = counter_peek(p.tag_src != nullptr ? p.tag_src : p.bar + kBarGen);
+    const int gen_lane = threadIdx.x & 63;
+    const int gen_word = counter_peek(p.tag_src != nullptr ? p.tag_src : group_counter(p.grp, kBarExit, gen_lane % kEventGroups));
     fused_layer<NCH, CPD, EX, BYX>(p, gen_word, lds);
 }
 
