@@ -498,7 +498,7 @@ def other_workloads(pkg, dev, args):
                 "value": r["value"], "unit": "ms/token", "bytes": r["step"]["bytes"], "hbm_gbps": r["step"]["hbm_gbps"],
                 "frac_of_peak": r["step"]["frac_of_peak"], "layer_kernel_us": r["roofline"]["layer_us"],
                 "layer_kernel_frac_of_peak": r["roofline"]["frac"], "sweep": r.get("sweep"),
-                "split_mode": r.get("split_mode")}
+                "launch_per_layer_mode": r.get("launch_per_layer_mode"), "split_mode": r.get("split_mode")}
 
     attempt("pythia_2b8 single layer (config 1)", lambda: single_layer("pythia_2b8", 512, 1))
     torch.cuda.empty_cache()
@@ -633,6 +633,23 @@ def main():
                                 "hbm_gbps": result["step"]["hbm_gbps"], "frac_of_peak": result["step"]["frac_of_peak"]}] + \
                 context_sweep(dec, cfg, stream, sweep_ctx)
         result["sweep"].sort(key=lambda r: r["context"])
+        try:
+            # the same model with one launch per layer (CFPP_MODE_FUSED_LAYERS): what the one launch for all layers is worth
+            ldec = pkg.NeoxDecoder(cfg, dec.tensors["layers"], dec.tensors["embed"], dec.tensors["final_ln_w"], dec.tensors["final_ln_b"],
+                                   dec.tensors["lm_head"], dec.tensors["k_caches"], dec.tensors["v_caches"], mode="fused_layers")
+            with torch.cuda.stream(stream):
+                lt = time_tokens(ldec, stream, args.ctx, 32, 6)
+            ldec.check()
+            lsb = step_bytes(cfg, args.ctx + 6 + 16)
+            result["launch_per_layer_mode"] = {"workload": f"{args.model} full stack, one fused launch per layer instead of one for all "
+                                                           f"layers, hipGraph replay, context {args.ctx}", "context": args.ctx, "tokens": 32,
+                                               "tpot_ms": round(lt, 4), "bytes": lsb, "hbm_gbps": round(lsb / (lt * 1e-3) / 1e9, 1),
+                                               "frac_of_peak": round(lsb / (lt * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+            log(f"[launch per layer] context {args.ctx}: {lt:.4f} ms/token = {result['launch_per_layer_mode']['frac_of_peak'] * 100:.1f} % of peak")
+            del ldec
+        except Exception as e:     # noqa: BLE001
+            log(f"[launch_per_layer_mode] failed: {type(e).__name__}: {e}")
+            result["launch_per_layer_mode"] = {"error": f"{type(e).__name__}: {e}"}
         try:
             # the same model through the per-stage launches (CFPP_MODE_SPLIT), sharing the weights and caches
             sdec = pkg.NeoxDecoder(cfg, dec.tensors["layers"], dec.tensors["embed"], dec.tensors["final_ln_w"], dec.tensors["final_ln_b"],
