@@ -2683,8 +2683,8 @@ LmTail stack_tail(const cfpp_neox_stack* s) {
     return LmTail{s->best_val, s->best_idx, s->state, s->state + kStateDone, s->history, s->hist_cap,
                   reinterpret_cast<const half_t*>(s->desc.embed), s->x0};
 }
-// one launch per layer and one for the LM head, whose last workgroup picks the token, advances the state and
-// fetches the picked token's embedding row for the next step
+// the layers (one launch for all of them, or one each), then the LM head, whose last workgroup picks the token, advances
+// the state and fetches the picked token's embedding row for the next step
 int stack_enqueue_step(cfpp_neox_stack* s, hipStream_t st) {
     const cfpp_neox_dims& d = s->desc.dims;
     const int rc = stack_enqueue_layers(s, st);
